@@ -50,6 +50,7 @@ LIBRARIES: Dict[str, tuple] = {
     "linear_attention": ("hip", ["hip/linear_attention.hip"], ["hip/common.h"]),
     "shortconv": ("hip", ["hip/shortconv.hip"], ["hip/common.h"]),
     "moe": ("hip", ["hip/moe.hip"], ["hip/common.h"]),
+    "headmix": ("hip", ["hip/headmix.hip"], ["hip/common.h"]),
 }
 
 _lock = threading.Lock()

@@ -3,6 +3,7 @@ from .base import (ConfigError, ModelConfig, architecture_of, config_from_dict, 
 from .llama import LlamaConfig
 from .sagalorn import SagalornConfig
 from .dekinex import DekinexConfig
+from .vumalix import VumalixConfig
 
-__all__ = ["ConfigError", "ModelConfig", "LlamaConfig", "SagalornConfig", "DekinexConfig", "architecture_of", "config_from_dict",
+__all__ = ["ConfigError", "ModelConfig", "LlamaConfig", "SagalornConfig", "DekinexConfig", "VumalixConfig", "architecture_of", "config_from_dict",
            "config_from_dir", "known_architectures", "lookup", "register_architecture"]

@@ -71,8 +71,25 @@ _SIGS = {
         # proj, dtype, stride, state, q_start, q_len, state slots, requests, channels, taps, stream
         "gb_conv_state": [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     },
-    "moe": {
-        # z, ldz, n, experts, correction, top, scale, shared, combine, ids, weights, stream
+    "headmix": {
+        # x, ldx, w, taps, state, tok_seq, q_start, pos0, state slots, out, dtype, ldo, n, d, single, stream
+        "gb_time_conv": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+        # in, dtype, ld, n, eps, (col, d, gamma, out, ldo) twice, stream
+        "gb_norm_slices": [_vp, _i, _i, _i, _f, _i, _i, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp],
+        # q, ldq, kv, ldkv, krot, ldr, dtype, cos, sin, rot, out, ldo, hd, slots, k, v, page, n, H, dim, rot_dim, vdim, stream
+        "gb_latent_heads": [_vp, _i, _vp, _i, _vp, _i, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+        # proj, dtype, ld, wq, wk, eps, coef, every, positions, out, ldo, hd, slots, k, v, page, n, H, G, dim, vdim, stream
+        "gb_diff_heads": [_vp, _i, _i, _vp, _vp, _f, _f, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+        # att, dtype, lda, hd, lambda, mult, eps, out, ldo, n, H, vdim, stream
+        "gb_diff_combine": [_vp, _i, _i, _i, _vp, _f, _f, _vp, _i, _i, _i, _i, _vp],
+        # att, lda, hd, gate, ldg, dtype, out, ldo, n, H, vdim, stream
+        "gb_gate_heads": [_vp, _i, _i, _vp, _i, _i, _vp, _i, _i, _i, _i, _vp],
+        # z, ldz, coef, eps, out, ldo, dtype, n, d, stream
+        "gb_poly_norm": [_vp, _i, _vp, _f, _vp, _i, _i, _i, _i, _vp],
+        # x, y, g, eps, rounded, dtype, n, d, stream
+        "gb_norm_add": [_vp, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+    },
+    "moe": {        # z, ldz, n, experts, correction, top, scale, shared, combine, ids, weights, stream
         "gb_moe_route": [_vp, _i, _i, _i, _vp, _i, _f, _i, _vp, _vp, _vp, _vp],
         # gate_up, its dtype, ld, combine, its columns, act, its dtype, n, inter, experts, ff, stream
         "gb_moe_gated_units": [_vp, _i, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
@@ -864,6 +881,180 @@ def conv_heads(proj: torch.Tensor, wconv: Optional[torch.Tensor], state: Optiona
     if wconv is not None and taps > 1 and not single:
         _launch(lib, lib.gb_conv_state, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(state), _p(ctx.q_start),
                 _p(ctx.q_len), _p(ctx.state_slots), ctx.num_seqs, channels, taps, _stream())
+
+
+# --------------------------------------------------------- sublayers with normed outputs; latent and differential heads
+TIME_CONV_MAX_TAPS = 8   # headmix.hip keeps a channel's slot in registers
+
+
+def _act_rows(t: torch.Tensor, dtype, cols: int, what: str) -> int:
+    """Row stride of a 2-d tensor of the activations' type with dense rows of at least ``cols`` columns."""
+    if t.dtype != dtype or t.dim() != 2 or t.stride(1) != 1 or t.shape[1] < cols:
+        raise KernelError(f"{what} must be 2-d {dtype} with dense rows of at least {cols} columns, got {tuple(t.shape)} {t.dtype}")
+    return t.stride(0)
+
+
+def time_conv(x: torch.Tensor, w: Optional[torch.Tensor], state: Optional[torch.Tensor], ctx, out: torch.Tensor) -> None:
+    """out = x + conv(x) in the type of ``out``: x float32 [n, d] (the residual), ``w`` float32 [d, taps] (None: out is x
+    rounded), conv(x)[t] = sum_j w[:, j] x[t - taps + 1 + j] over the request's own tokens, zeros before its first.  The
+    request's last taps - 1 rows of x live in ``state`` (float32 [slots, taps - 1, d]) and are moved on by this call, so
+    it must come before x changes."""
+    _dev(x, w, state, out)
+    n, d = x.shape
+    _f32_rows(x, (n, d), "x")
+    taps = 0
+    if w is not None:
+        taps = w.shape[1]
+        _f32_rows(w, (d, taps), "w")
+        if taps > TIME_CONV_MAX_TAPS:
+            raise KernelError(f"time_conv: {taps} taps are above {TIME_CONV_MAX_TAPS}")
+        if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
+                         or tuple(state.shape[1:]) != (taps - 1, d)):
+            raise KernelError("time_conv: state must be contiguous float32 [slots, taps - 1, d]")
+    ldo = _act_rows(out, out.dtype, d, "out")
+    if out.shape[0] != n:
+        raise KernelError("time_conv: out must have x's rows")
+    single = int(ctx.host["max_q_len"]) == 1
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_time_conv, _p(x), x.stride(0), _p(w), taps, _p(state) if taps > 1 else None, _p(ctx.tok_seq),
+            _p(ctx.q_start), _p(ctx.pos0), _p(ctx.state_slots), _p(out), dtype_code(out), ldo, n, d, 1 if single else 0,
+            _stream())
+    if taps > 1 and not single:
+        conv = _lib("shortconv")
+        _launch(conv, conv.gb_conv_state, _p(x), F32, x.stride(0), _p(state), _p(ctx.q_start), _p(ctx.q_len),
+                _p(ctx.state_slots), ctx.num_seqs, d, taps, _stream())
+
+
+def norm_slices(rows: torch.Tensor, eps: float, first, second=None) -> None:
+    """RMS norms with a weight over runs of columns of ``rows``: ``first`` and ``second`` are (column, gamma float32 [d],
+    out [n, >= d] of the rows' type); out = gamma * v / sqrt(mean(v^2) + eps) over the run's d columns."""
+    n = rows.shape[0]
+    ld = _act_rows(rows, rows.dtype, 1, "rows")
+    args = []
+    for item in (first, second):
+        if item is None:
+            args += [0, 0, None, None, 0]
+            continue
+        col, gamma, out = item
+        d = gamma.numel()
+        _dev(rows, gamma, out)
+        _f32_rows(gamma, (d,), "gamma")
+        if col < 0 or col + d > rows.shape[1] or out.shape[0] != n:
+            raise KernelError("norm_slices: a run of columns beyond the rows")
+        args += [int(col), d, _p(gamma), _p(out), _act_rows(out, rows.dtype, d, "out")]
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_norm_slices, _p(rows), dtype_code(rows), ld, n, float(eps), *args, _stream())
+
+
+def _store_args(slots, k_pages, v_pages, dtype, n: int, kv_heads: int, head_cols: int, what: str):
+    if slots is None:
+        return None, None, None, 0
+    _dev(slots, k_pages, v_pages)
+    _i32(slots, "slots", n)
+    _, p_heads, page_size, p_hd = _check_pages(k_pages, v_pages, dtype, what)
+    if (p_heads, p_hd) != (kv_heads, head_cols):
+        raise KernelError(f"{what}: pages do not have this layer's kv heads and head size")
+    return _p(slots), _p(k_pages), _p(v_pages), page_size
+
+
+def latent_heads(q: torch.Tensor, kv: torch.Tensor, k_rot: torch.Tensor, cos: Optional[torch.Tensor],
+                 sin: Optional[torch.Tensor], rot: int, out: torch.Tensor, head_cols: int, slots: Optional[torch.Tensor],
+                 k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, dim: int, rot_dim: int,
+                 vdim: int) -> None:
+    """Heads for attention through latents.  ``q`` [n, heads * (dim + rot_dim)]; ``kv`` [n, heads * dim + heads * vdim] (the
+    heads' own key parts, then their values); ``k_rot`` [n, rot_dim], the key part all heads share.  The first ``rot`` of
+    the rot_dim columns of every query head and of the shared part are turned in half-split pairs (i, i + rot / 2) by
+    the rows' angles (``cos``, ``sin`` float32 [n, rot / 2]).  ``out`` [n, 3 * heads * head_cols]: query heads, key heads
+    [own part | shared part], value heads, each filled up with zeros; with ``slots`` keys and values also go to the pages."""
+    _dev(q, kv, k_rot, cos, sin, out)
+    n, dt = q.shape[0], q.dtype
+    ldq = _act_rows(q, dt, n_heads * (dim + rot_dim), "q")
+    ldkv = _act_rows(kv, dt, n_heads * (dim + vdim), "kv")
+    ldr = _act_rows(k_rot, dt, rot_dim, "k_rot") if rot_dim else max(1, k_rot.stride(0))
+    ldo = _act_rows(out, dt, 3 * n_heads * head_cols, "out")
+    if rot:
+        for t in (cos, sin):
+            if t is None or t.dtype != torch.float32 or not t.is_contiguous() or t.shape[1] != rot // 2 or t.shape[0] < n:
+                raise KernelError("latent_heads: cos/sin must be contiguous float32 [n, rot / 2]")
+    store = _store_args(slots, k_pages, v_pages, dt, n, n_heads, head_cols, "latent_heads")
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_latent_heads, _p(q), ldq, _p(kv), ldkv, _p(k_rot), ldr, dtype_code(q), _p(cos) if rot else None,
+            _p(sin) if rot else None, int(rot), _p(out), ldo, int(head_cols), *store, n, n_heads, dim, rot_dim, vdim, _stream())
+
+
+def diff_heads(proj: torch.Tensor, w_q: torch.Tensor, w_k: torch.Tensor, eps: float, coef: float, every: int,
+               positions: torch.Tensor, out: torch.Tensor, head_cols: int, slots: Optional[torch.Tensor],
+               k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, dim: int,
+               vdim: int) -> None:
+    """Heads for differential attention.  ``proj`` [n, heads * 2 dim + kv heads * 2 dim + kv heads * vdim]: every query
+    and key head holds two maps of dim columns.  Each map is divided by its root mean square and multiplied by ``w_q``
+    (``w_k``), float32 [dim]; query maps also by 1 + coef * ln(floor((position + 1) / every) + 1) (``every`` 0: not).
+    ``out`` [n, (2 heads + 2 kv heads) * head_cols]: query heads [q1 | 0], [0 | q2] for each head, key heads [k1 | k2],
+    value heads, filled up with zeros; with ``slots`` keys and values also go to the pages (kv heads of head_cols)."""
+    _dev(proj, w_q, w_k, positions, out)
+    n, dt = proj.shape[0], proj.dtype
+    ld = _act_rows(proj, dt, (n_heads + n_kv_heads) * 2 * dim + n_kv_heads * vdim, "proj")
+    ldo = _act_rows(out, dt, (2 * n_heads + 2 * n_kv_heads) * head_cols, "out")
+    _f32_rows(w_q, (dim,), "w_q")
+    _f32_rows(w_k, (dim,), "w_k")
+    _i32(positions, "positions", n)
+    store = _store_args(slots, k_pages, v_pages, dt, n, n_kv_heads, head_cols, "diff_heads")
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_diff_heads, _p(proj), dtype_code(proj), ld, _p(w_q), _p(w_k), float(eps), float(coef), int(every),
+            _p(positions), _p(out), ldo, int(head_cols), *store, n, n_heads, n_kv_heads, dim, vdim, _stream())
+
+
+def diff_combine(att: torch.Tensor, head_cols: int, lam: torch.Tensor, mult: float, eps: float, out: torch.Tensor,
+                 n_heads: int, vdim: int) -> None:
+    """out[:, h] = mult * o / sqrt(mean(o^2) + eps), o = a1 - lam * a2, where a1, a2 are heads 2 h and 2 h + 1 of ``att``
+    ([n, 2 heads * head_cols]) cut to vdim columns and ``lam`` is one float32 on the device; ``out`` [n, heads * vdim]."""
+    _dev(att, lam, out)
+    n, dt = att.shape[0], att.dtype
+    lda = _act_rows(att, dt, 2 * n_heads * head_cols, "att")
+    ldo = _act_rows(out, dt, n_heads * vdim, "out")
+    _f32_rows(lam, (1,), "lam")
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_diff_combine, _p(att), dtype_code(att), lda, int(head_cols), _p(lam), float(mult), float(eps),
+            _p(out), ldo, n, n_heads, vdim, _stream())
+
+
+def gate_heads(att: torch.Tensor, head_cols: int, gate: torch.Tensor, out: torch.Tensor, n_heads: int, vdim: int) -> None:
+    """out[:, h, c] = att[:, h, c] * sigmoid(gate[:, h, c]) for c < vdim: ``att`` [n, heads * head_cols], ``gate`` and
+    ``out`` [n, heads * vdim]."""
+    _dev(att, gate, out)
+    n, dt = att.shape[0], att.dtype
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_gate_heads, _p(att), _act_rows(att, dt, n_heads * head_cols, "att"), int(head_cols), _p(gate),
+            _act_rows(gate, dt, n_heads * vdim, "gate"), dtype_code(att), _p(out), _act_rows(out, dt, n_heads * vdim, "out"),
+            n, n_heads, vdim, _stream())
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e over every row, powers element by element, N(v) = v / sqrt(mean(v^2) + eps);
+    ``coef`` float32 [4] = a, b, c, e."""
+    _dev(z, coef, out)
+    n, d = z.shape
+    _f32_rows(coef, (4,), "coef")
+    if out.shape != z.shape:
+        raise KernelError("poly_norm: out must have z's shape")
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_poly_norm, _p(z), _act_rows(z, z.dtype, d, "z"), _p(coef), float(eps), _p(out),
+            _act_rows(out, z.dtype, d, "out"), dtype_code(z), n, d, _stream())
+
+
+def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, rounded: Optional[torch.Tensor] = None) -> None:
+    """x += g * y / sqrt(mean(y^2) + eps) row by row: x, y float32 [n, d], ``g`` one float32 on the device.  ``rounded``
+    ([n, d], any activations' type) receives the new x."""
+    _dev(x, y, g, rounded)
+    n, d = x.shape
+    _f32_rows(x, (n, d), "x")
+    _f32_rows(y, (n, d), "y")
+    _f32_rows(g, (1,), "g")
+    if rounded is not None and (tuple(rounded.shape) != (n, d) or not rounded.is_contiguous()):
+        raise KernelError("norm_add: rounded must be contiguous [n, d]")
+    lib = _lib("headmix")
+    _launch(lib, lib.gb_norm_add, _p(x), _p(y), _p(g), float(eps), _p(rounded),
+            dtype_code(rounded) if rounded is not None else F32, n, d, _stream())
 
 
 # ------------------------------------------------------------------- routed experts

@@ -332,3 +332,176 @@ class ShortConvAttention(Mixer):
         att = ctx.buffer("att", (n, H * hc), ctx.dtype)
         paged_attention(ctx, heads[:, :H * hc], att, cache, H, self.scale, self.window)
         product(ctx, att, self.wo, residual, accumulate=not store)
+
+
+def _stack_rows(parts, width: int) -> torch.Tensor:
+    """Matrices stacked by rows into one product, filled up with zero rows to a multiple of 8 (rows of the product's
+    result then begin at 16-byte words)."""
+    parts = list(parts)
+    rows = sum(p.shape[0] for p in parts)
+    if rows % 8:
+        parts.append(torch.zeros((8 - rows % 8, width), dtype=parts[0].dtype, device=parts[0].device))
+    return torch.cat(parts, 0)
+
+
+class LatentAttention(Mixer):
+    """Attention whose queries, keys and values come through narrow latents.  c_q = norm(W_dq h) (RMS norm with a weight),
+    q = W_uq c_q, every query head [dim columns as they are | rot_dim columns that are rotated].  W_dkv h has kv_rank + rot_dim
+    rows: the first kv_rank, normed with a weight, are the latent c; the last rot_dim, not normed, are one rotated key part
+    that all heads share.  A head's key is [W_uk c | the shared part], its value W_uv c; scores q . k * scale over the last
+    ``window`` keys (0: all); softmax.  The first ``rot_dims`` of the rot_dim columns turn with the position in half-split
+    pairs (i, i + rot_dims / 2), frequencies base^(-2i / rot_dims).  The heads are multiplied by sigmoid(W_g h) before the
+    output projection.
+
+    Tensors: ``dq``, ``dq.norm``, ``uq``, ``dkv``, ``dkv.norm``, ``uk``, ``uv``, ``g``, ``o``.  The pages hold every head's key
+    and value as attention reads them (heads of ``cache_head_cols(dim + rot_dim, vdim)`` columns)."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, n_heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int, scale: float,
+                 window: int = 0, rot_dims: Optional[int] = None, rot_base: float = 10000.0, eps: float = 1e-5):
+        from .rotary import Rotary
+        rot_dims = rot_dim if rot_dims is None else rot_dims
+        if rot_dims % 2 or not 0 <= rot_dims <= rot_dim:
+            raise ValueError(f"{rot_dims} rotated columns: an even number up to rot_dim {rot_dim}")
+        self.width, self.n_heads, self.dim, self.rot_dim, self.vdim = width, n_heads, dim, rot_dim, vdim
+        self.q_rank, self.kv_rank = q_rank, kv_rank
+        self.scale, self.window, self.rot_dims, self.eps = float(scale), int(window), int(rot_dims), float(eps)
+        self.head_cols = cache_head_cols(dim + rot_dim, vdim)
+        self.position = Rotary(rot_dims, rot_base) if rot_dims else None
+        self.cache_spec = CacheSpec(n_heads, self.head_cols, WINDOW if window > 0 else FULL, self.window)
+        self.w_in = self.w_uq = self.w_ukv = self.wo = self.norm_q = self.norm_kv = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        H, D, R, V = self.n_heads, self.dim, self.rot_dim, self.vdim
+        return {"dq": TensorSpec((self.q_rank, self.width)), "dq.norm": TensorSpec((self.q_rank,), kind="f32", init="ones"),
+                "uq": TensorSpec((H * (D + R), self.q_rank)),
+                "dkv": TensorSpec((self.kv_rank + R, self.width)), "dkv.norm": TensorSpec((self.kv_rank,), kind="f32", init="ones"),
+                "uk": TensorSpec((H * D, self.kv_rank)), "uv": TensorSpec((H * V, self.kv_rank)),
+                "g": TensorSpec((H * V, self.width)), "o": TensorSpec((self.width, H * V))}
+
+    def load(self, tensors):
+        # one product reads the mixer's input for both latents, the shared key part and the gate
+        self.w_in = _stack_rows([tensors["dq"], tensors["dkv"], tensors["g"]], self.width)
+        self.w_uq = tensors["uq"].contiguous()
+        self.w_ukv = _stack_rows([tensors["uk"], tensors["uv"]], self.kv_rank)
+        self.wo = tensors["o"].contiguous()
+        self.norm_q, self.norm_kv = tensors["dq.norm"].float().contiguous(), tensors["dkv.norm"].float().contiguous()
+
+    def streamed_matrices(self):
+        return [self.w_in, self.w_uq, self.w_ukv, self.wo]
+
+    def problems(self, dtype, page_size):
+        if self.head_cols > ops.MAX_HEAD_DIM:
+            return [("dim", f"heads of {max(self.dim + self.rot_dim, self.vdim)} columns are above {ops.MAX_HEAD_DIM}, the "
+                            f"largest head the attention kernels take")]
+        return []
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
+        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        if cache is None or cache.k_pages is None:
+            raise ValueError("LatentAttention needs a layer cache with pages")
+        n = h.shape[0]
+        H, D, R, V, hc = self.n_heads, self.dim, self.rot_dim, self.vdim, self.head_cols
+        first = ctx.buffer("latent_in", (n, self.w_in.shape[0]), ctx.dtype)     # [c_q | c | shared key part | gate]
+        product(ctx, h, self.w_in, first)
+        c_q = ctx.buffer("latent_cq", (n, self.q_rank), ctx.dtype)
+        c_kv = ctx.buffer("latent_ckv", (n, self.kv_rank), ctx.dtype)
+        ops.norm_slices(first, self.eps, (0, self.norm_q, c_q), (self.q_rank, self.norm_kv, c_kv))
+        q = ctx.buffer("latent_q", (n, self.w_uq.shape[0]), ctx.dtype)
+        product(ctx, c_q, self.w_uq, q)
+        kv = ctx.buffer("latent_kv", (n, self.w_ukv.shape[0]), ctx.dtype)
+        product(ctx, c_kv, self.w_ukv, kv)
+        cos, sin = self.position.table(ctx) if self.position is not None else (None, None)
+        heads = ctx.buffer("latent_heads", (n, 3 * H * hc), ctx.dtype)
+        slots = ctx.slots[cache.group] if cache.writable else None
+        direct = slots is not None and n <= ops.ROPE_PRODUCT_MAX_ROWS
+        shared = self.q_rank + self.kv_rank
+        ops.latent_heads(q, kv, first[:, shared:shared + max(R, 1)], cos, sin, self.rot_dims, heads, hc,
+                         slots if direct else None, cache.k_pages, cache.v_pages, H, D, R, V)
+        if slots is not None and not direct:
+            # many rows: the kernel that takes a step's keys and values to their pages in whole lines
+            ops.rope_store(heads, None, None, slots, cache.k_pages, cache.v_pages, H, H, hc, rotate=False,
+                           portions=ctx.portions())
+        att = ctx.buffer("att", (n, H * hc), ctx.dtype)
+        paged_attention(ctx, heads[:, :H * hc], att, cache, H, self.scale, self.window)
+        gated = ctx.buffer("latent_gated", (n, H * V), ctx.dtype)
+        ops.gate_heads(att, hc, first[:, shared + R:shared + R + H * V], gated, H, V)
+        product(ctx, gated, self.wo, residual, accumulate=not store)
+
+
+class DifferentialAttention(Mixer):
+    """Grouped-query attention with two softmax maps a head over the same values: every query and key head holds two
+    maps of ``dim`` columns, [map 1 | map 2]; each map is divided by its root mean square and multiplied by a weight of
+    dim numbers (``q.norm``, ``k.norm``, shared by all heads and maps); query maps are also multiplied by the
+    temperature 1 + coef * ln(floor((position + 1) / every) + 1) (``temp_every`` 0: not); scores q . k * scale over all
+    earlier keys; positions enter nowhere else.  With a1, a2 the maps' outputs, o = a1 - lambda a2, lambda =
+    exp(lq1 . lk1) - exp(lq2 . lk2) + diff (one number for the layer), then o / sqrt(mean(o^2) + eps) * (1 - diff) over
+    the head's vdim values, and the output projection.
+
+    The two maps of a head are run as two query heads of 2 dim columns, [q1 | 0] and [0 | q2], over one key head
+    [k1 | k2]: the zeros leave each map its own score, and both read the same cached values.
+
+    Tensors: ``q``, ``k``, ``v``, ``q.norm``, ``k.norm``, ``lq1``, ``lk1``, ``lq2``, ``lk2``, ``o``."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: float, diff: float,
+                 temp_coef: float = 0.0, temp_every: int = 0, eps: float = 1e-5):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key heads")
+        self.width, self.n_heads, self.n_kv_heads, self.dim, self.vdim = width, n_heads, n_kv_heads, dim, vdim
+        self.scale, self.diff, self.eps = float(scale), float(diff), float(eps)
+        self.temp_coef, self.temp_every = float(temp_coef), int(temp_every)
+        self.head_cols = cache_head_cols(2 * dim, vdim)
+        self.cache_spec = CacheSpec(n_kv_heads, self.head_cols, FULL, 0)
+        self.wqkv = self.wo = self.norm_q = self.norm_k = self.lam = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        H, G, D, V = self.n_heads, self.n_kv_heads, self.dim, self.vdim
+        specs = {"q": TensorSpec((H * 2 * D, self.width)), "k": TensorSpec((G * 2 * D, self.width)),
+                 "v": TensorSpec((G * V, self.width)), "o": TensorSpec((self.width, H * V)),
+                 "q.norm": TensorSpec((D,), kind="f32", init="ones"), "k.norm": TensorSpec((D,), kind="f32", init="ones")}
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            specs[name] = TensorSpec((D,), kind="f32")
+        return specs
+
+    def load(self, tensors):
+        self.wqkv = _stack_rows([tensors["q"], tensors["k"], tensors["v"]], self.width)
+        self.wo = tensors["o"].contiguous()
+        self.norm_q, self.norm_k = tensors["q.norm"].float().contiguous(), tensors["k.norm"].float().contiguous()
+        one, two = (tensors["lq1"].float() * tensors["lk1"].float()).sum(), (tensors["lq2"].float() * tensors["lk2"].float()).sum()
+        self.lam = (torch.exp(one) - torch.exp(two) + self.diff).reshape(1).contiguous()   # a number of the weights alone
+
+    def streamed_matrices(self):
+        return [self.wqkv, self.wo]
+
+    def problems(self, dtype, page_size):
+        if self.head_cols > ops.MAX_HEAD_DIM:
+            return [("dim", f"heads of {max(2 * self.dim, self.vdim)} columns (two maps of dim) are above {ops.MAX_HEAD_DIM}, "
+                            f"the largest head the attention kernels take")]
+        return []
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
+        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        if cache is None or cache.k_pages is None:
+            raise ValueError("DifferentialAttention needs a layer cache with pages")
+        n = h.shape[0]
+        H, G, V, hc = self.n_heads, self.n_kv_heads, self.vdim, self.head_cols
+        proj = ctx.buffer("diff_proj", (n, self.wqkv.shape[0]), ctx.dtype)
+        product(ctx, h, self.wqkv, proj)
+        heads = ctx.buffer("diff_heads", (n, (2 * H + 2 * G) * hc), ctx.dtype)
+        slots = ctx.slots[cache.group] if cache.writable else None
+        direct = slots is not None and n <= ops.ROPE_PRODUCT_MAX_ROWS
+        ops.diff_heads(proj, self.norm_q, self.norm_k, self.eps, self.temp_coef, self.temp_every, ctx.positions, heads, hc,
+                       slots if direct else None, cache.k_pages, cache.v_pages, H, G, self.dim, V)
+        if slots is not None and not direct:
+            ops.rope_store(heads, None, None, slots, cache.k_pages, cache.v_pages, 2 * H, G, hc, rotate=False,
+                           portions=ctx.portions())
+        att = ctx.buffer("att", (n, 2 * H * hc), ctx.dtype)
+        paged_attention(ctx, heads[:, :2 * H * hc], att, cache, 2 * H, self.scale, 0)
+        o = ctx.buffer("diff_o", (n, H * V), ctx.dtype)
+        ops.diff_combine(att, hc, self.lam, 1.0 - self.diff, self.eps, o, H, V)
+        product(ctx, o, self.wo, residual, accumulate=not store)

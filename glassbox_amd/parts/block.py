@@ -128,3 +128,57 @@ class ParallelBlock(Block):
             self.ffn.forward(ctx, h, y)
         ops.axpy_rows(x, y, self.mult)
         return None
+
+
+class OutputNormBlock(Block):
+    """A layer that norms what its sublayers give back, not what they read: x += norm1(mixer(conv(x))), then
+    x += norm2(feed-forward(x)); the
+    feed-forward may be absent.  The sublayers read the residual itself (the mixer through ``conv``, which may add a short
+    convolution of the residual over time and keeps the state that takes); each writes its rows into a 32-bit buffer
+    (``accepts_store``), and the norm's pass over them is the pass that adds them into the residual.  The norms are
+    ``ScalarRMSNorm``s (or anything with ``add_normed``)."""
+    replayable = True
+    taped = True
+
+    def __init__(self, conv, mixer: Mixer, mixer_norm, ffn: Optional[FeedForward] = None, ffn_norm=None,
+                 names=("canon1", "mix", "norm1", "mlp", "norm2")):
+        for part in (mixer, ffn):
+            if part is not None and not getattr(part, "accepts_store", False):
+                raise ValueError(f"{type(part).__name__} cannot write its rows instead of adding them (accepts_store)")
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        if conv.state_spec is not None and mixer.state_spec is not None:
+            raise ValueError("the convolution and the mixer both keep state: a cache layer has one state")
+        self.conv, self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = conv, mixer, mixer_norm, ffn, ffn_norm
+        self.names = tuple(names)
+
+    def children(self) -> Dict[str, Part]:
+        out = {self.names[0]: self.conv, self.names[1]: self.mixer, self.names[2]: self.mixer_norm}
+        if self.ffn is not None:
+            out[self.names[3]] = self.ffn
+            out[self.names[4]] = self.ffn_norm
+        return out
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return self.mixer.cache_spec
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return self.conv.state_spec if self.conv.state_spec is not None else self.mixer.state_spec
+
+    def forward(self, ctx, x, cache: Optional[LayerCache]):
+        n, width = x.shape
+        h = self.conv.forward(ctx, x, cache)
+        y = ctx.buffer("sublayer_y", (n, width), torch.float32)
+        self.mixer.forward(ctx, h, y, cache, store=True)
+        if self.ffn is None:
+            self.mixer_norm.add_normed(ctx, y, x)
+            return None
+        if ctx.dtype == torch.float32:
+            self.mixer_norm.add_normed(ctx, y, x)
+            rows = x
+        else:   # the pass that makes the residual also leaves it in the activations' type for the feed-forward
+            rows = ctx.buffer("h", (n, width), ctx.dtype)
+            self.mixer_norm.add_normed(ctx, y, x, rounded=rows)
+        self.ffn.forward(ctx, rows, y, store=True)
+        self.ffn_norm.add_normed(ctx, y, x)
+        return None

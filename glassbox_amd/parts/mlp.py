@@ -113,3 +113,36 @@ class ClampedGLU(FeedForward):
             ops.glu_clamped(gate_up, act, self.limit, self.alpha)
         product(ctx, act, self.w_down, residual, accumulate=not store)
         return None
+
+
+class PolyNormMLP(FeedForward):
+    """W_down act(W_up h) without a gate; act is a polynomial of normed powers, a N(z) + b N(z^2) + c N(z^3) + e with
+    the powers taken element by element and N(v) = v / sqrt(mean(v^2) + eps) over a token's ``intermediate`` values;
+    ``act`` holds a, b, c, e.  The sums are 32-bit."""
+    replayable = True
+    taped = True
+    accepts_store = True
+
+    def __init__(self, width: int, intermediate: int, eps: float):
+        self.width, self.intermediate, self.eps = width, intermediate, float(eps)
+        self.w_up = self.w_down = self.coef = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {"up": TensorSpec((self.intermediate, self.width)), "down": TensorSpec((self.width, self.intermediate)),
+                "act": TensorSpec((4,), kind="f32", init="ones")}
+
+    def load(self, tensors):
+        self.w_up, self.w_down = tensors["up"].contiguous(), tensors["down"].contiguous()
+        self.coef = tensors["act"].float().contiguous()
+
+    def streamed_matrices(self):
+        return [self.w_up, self.w_down]
+
+    def forward(self, ctx, h, residual, store: bool = False):
+        n = h.shape[0]
+        z = ctx.buffer("poly_z", (n, self.intermediate), ctx.dtype)
+        product(ctx, h, self.w_up, z)
+        act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
+        ops.poly_norm(z, self.coef, self.eps, act)
+        product(ctx, act, self.w_down, residual, accumulate=not store)
+        return None

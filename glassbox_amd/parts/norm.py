@@ -1,6 +1,7 @@
 """RMS norm: out = g * (x / sqrt(mean(x^2) + eps)), sums in 32-bit
 (crates/glassbox-core/src/model.rs:94-100).  With ``offset`` the checkpoint holds the weight minus ``offset`` and
-g = offset + w, added in 32-bit when the weights are loaded and kept in 32-bit."""
+g = offset + w, added in 32-bit when the weights are loaded and kept in 32-bit.  ``ScalarRMSNorm`` has one number for all
+coordinates and can also norm a sublayer's *output* on its way into the residual."""
 from __future__ import annotations
 
 from typing import Dict, Optional, Tuple
@@ -49,3 +50,34 @@ class RMSNorm(Norm):
         if ctx.dtype == torch.bfloat16 and n <= ops.FUSED_NORM_MAX_ROWS and ctx.fuse_norms:
             return (self.weight, self.eps)
         return None
+
+
+class ScalarRMSNorm(Norm):
+    """out = g * (x / sqrt(mean(x^2) + eps)) with a single number g (a tensor without dimensions).  As a norm of rows
+    (``forward``: a final norm) it is the kernel of ``RMSNorm`` with g in every column; ``add_normed`` norms a
+    sublayer's output y and adds it into the residual in one pass."""
+    replayable = True
+    taped = True
+
+    def __init__(self, width: int, eps: float):
+        self.width = width
+        self.eps = float(eps)
+        self.gain: Optional[torch.Tensor] = None      # [1]
+        self.weight: Optional[torch.Tensor] = None    # [width], the same number
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {"weight": TensorSpec((), kind="f32", init="ones")}
+
+    def load(self, tensors):
+        self.gain = tensors["weight"].float().reshape(1).contiguous()
+        self.weight = self.gain.expand(self.width).contiguous()
+
+    def forward(self, ctx, x, rows=None, out_name="h"):
+        m = x.shape[0] if rows is None else rows.numel()
+        out = ctx.buffer(out_name, (m, self.width), ctx.dtype)
+        ops.rmsnorm(x, self.weight, self.eps, out, rows)
+        return out
+
+    def add_normed(self, ctx, y, x, rounded=None) -> None:
+        """x += g * y / sqrt(mean(y^2) + eps) (both float32); ``rounded`` receives the new x in its own type."""
+        ops.norm_add(x, y, self.gain, self.eps, rounded)

@@ -53,12 +53,12 @@ def read_safetensors(path: str) -> Dict[str, torch.Tensor]:
     for name, e in header.items():
         b, end = e["data_offsets"]
         arr = np.frombuffer(data, dtype=kinds[e["dtype"]], count=(end - b) // np.dtype(kinds[e["dtype"]]).itemsize,
-                            offset=8 + n + b).reshape(e["shape"])
+                            offset=8 + n + b)
         if e["dtype"] == "BF16":
             # a bfloat16 is the upper half of a float32 (load.rs:23-26 converts to f32)
-            t = torch.from_numpy((arr.astype(np.uint32) << 16).view(np.float32).copy())
+            t = torch.from_numpy((arr.astype(np.uint32) << 16).view(np.float32).copy()).reshape(e["shape"])
         else:
-            t = torch.from_numpy(arr.astype(np.float64 if e["dtype"] == "F64" else np.float32).copy())
+            t = torch.from_numpy(arr.astype(np.float64 if e["dtype"] == "F64" else np.float32).copy()).reshape(e["shape"])
         out[name] = t
     return out
 
