@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
                     [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
-    python bench.py --design sagalorn|dekinex [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
+    python bench.py --design sagalorn|dekinex|vumalix [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
 
 ``--design sagalorn`` is another measurement with a line of its own: prefill and decode throughput of Sagalorn models
 whose layers have the sizes of the named shapes (a third of the layers each retention, windowed attention with kept
@@ -15,6 +15,12 @@ head rotated, a window of 1,024) and the matrix memory with exponential gates in
 clamped halves in every other layer and routed experts in the rest (eight experts of a quarter of the dense size, two a
 token, and a shared one of half the dense size: as many multiply-adds a token as the dense layer), a pair table of
 65,536 rows.
+
+``--design vumalix`` does the same for Vumalix models: two layers of attention through latents (heads of the Llama's head
+size plus half as many rotated columns, a query latent of 3/8 and a key/value latent of 1/4 of the width, a window of
+1,024) to one of differential attention (two maps of half the head size a head), every mixer behind a convolution of
+the residual over four tokens, every layer with a polynomial feed-forward of one and a half times the Llama's
+intermediate size (two matrices where the Llama has three: the same bytes and multiply-adds).
 
 A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step``
 (which replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the
@@ -90,7 +96,23 @@ def dekinex_like(shapes: dict, layers: int, window: int = 1024, experts: int = 8
                 layers=[kinds[i % 4] for i in range(layers)])
 
 
-DESIGNS = {"sagalorn": ("Sagalorn", sagalorn_like), "dekinex": ("Dekinex", dekinex_like)}
+def vumalix_like(shapes: dict, layers: int, window: int = 1024) -> dict:
+    """A Vumalix configuration with the widths of a Llama one: two latent-attention layers to one of differential
+    attention, a feed-forward of two matrices with the bytes of the Llama's three."""
+    d, H, G = shapes["hidden_size"], shapes["num_attention_heads"], shapes["num_key_value_heads"]
+    hd = shapes.get("head_dim") or d // H
+    mlp = {"kind": "dense", "ff": shapes["intermediate_size"] * 3 // 2 // 8 * 8}
+    latent = {"heads": H, "dim": hd, "rot_dim": hd // 2, "vdim": hd, "q_rank": d * 3 // 8 // 8 * 8, "kv_rank": d // 4 // 8 * 8,
+              "scale": (hd + hd // 2) ** -0.5, "rot": {"dims": hd // 2, "base": 10000.0}, "mask": {"size": window}}
+    diff = {"heads": H, "kv_heads": G, "dim": hd // 2, "vdim": hd, "scale": (hd // 2) ** -0.5, "diff": 0.6,
+            "q_temp": {"coef": 0.3, "every": 256}}
+    kinds = [{"type": "latent_attention", "mixer": latent, "mlp": mlp}, {"type": "latent_attention", "mixer": latent, "mlp": mlp},
+             {"type": "attention", "mixer": diff, "mlp": mlp}]
+    return dict(architecture="Vumalix", vocab=shapes["vocab_size"], width=d, norm={"eps": shapes["rms_norm_eps"]}, canon={"taps": 4},
+                layers=[kinds[i % 3] for i in range(layers)])
+
+
+DESIGNS = {"sagalorn": ("Sagalorn", sagalorn_like), "dekinex": ("Dekinex", dekinex_like), "vumalix": ("Vumalix", vumalix_like)}
 
 
 def design_bench(a) -> int:

@@ -81,6 +81,14 @@ def rotate_half_split(x: torch.Tensor, positions: torch.Tensor, base: float) -> 
     return torch.cat([u * cs - v * sn, v * cs + u * sn], -1)
 
 
+def rotate_first(x: torch.Tensor, positions: torch.Tensor, rot: Optional[dict]) -> torch.Tensor:
+    """The first rot["dims"] of the last dimension turn, the rest pass unchanged."""
+    if not rot or not rot["dims"]:
+        return x
+    n = rot["dims"]
+    return torch.cat([rotate_half_split(x[..., :n], positions, rot["base"]), x[..., n:]], -1)
+
+
 # ---------------------------------------------------------------------------------------------- softmax attention
 def visible(T: int, window: int = 0) -> torch.Tensor:
     """[T, T] truth values: query i sees key j if j <= i and, with a window, i - j < window."""
@@ -111,8 +119,8 @@ def latent_attention(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exac
     q = rnd(cq @ w[pre + "uq"].T).view(T, H, dk + dr)
     down = rnd(h @ w[pre + "dkv"].T)
     c = rnd(unit_rms(down[:, :rank], eps) * w[pre + "dkv.norm"])
-    k_rot = rotate_half_split(down[:, rank:], pos, m["rot"]["base"])                  # [T, dr], one for all heads
-    q_rot = rotate_half_split(q[..., dk:], pos, m["rot"]["base"])
+    k_rot = rotate_first(down[:, rank:], pos, m.get("rot"))                  # [T, dr], one for all heads
+    q_rot = rotate_first(q[..., dk:], pos, m.get("rot"))
     k_flat = rnd(c @ w[pre + "uk"].T).view(T, H, dk)
     v = rnd(c @ w[pre + "uv"].T).view(T, H, dv)
     qq = rnd(torch.cat([q[..., :dk], q_rot], -1))
