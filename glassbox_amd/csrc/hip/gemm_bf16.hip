@@ -1073,7 +1073,8 @@ inline int emit_parts(int M, int N) {
 
 template <int EPI, typename CT>
 int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc, int M, int N, int K, float* ws,
-                 const SplitPlan& plan, hipStream_t stream, const NormExtras* norm = nullptr, float eps = 0.f) {
+                 const SplitPlan& plan, hipStream_t stream, const NormExtras* norm = nullptr, float eps = 0.f,
+                 bool second_pass = true) {
   const dim3 grid((N + 127) / 128, (M + plan.bm - 1) / plan.bm, plan.slices), block(256);
   const bool kfull = K % TBK == 0;
   const bool ring = plan.ring && ring_takes(a, lda, w, ldw, K);
@@ -1091,6 +1092,7 @@ int launch_split(const bf16* a, int lda, const bf16* w, int ldw, CT* c, int ldc,
   GB_S(1, true) GB_S(1, false) GB_S(2, true) GB_S(2, false)
 #undef GB_S
   if (int rc = launched("gemm_bf16 (split k)")) return rc;
+  if (!second_pass) return 0;   // the caller adds the slices
   if constexpr (EPI == EPI_ACCUMULATE && std::is_same<CT, float>::value) {
     if (norm && norm->emit_h) {
       if (norm->emit_gamma_f32)
@@ -1731,6 +1733,29 @@ extern "C" long long gb_gemm_bf16_split_floats(int M, int N, int K) {
   return M > 16 ? (long long)split_plan(M, N, K).floats : 0;
 }
 
+// Slices into which gb_gemm_bf16_partial divides k for a product of these sizes (1: it would not divide it).
+extern "C" int gb_gemm_bf16_slices(int M, int N, int K) {
+  if (M <= 16) return 1;
+  const SplitPlan plan = split_plan(M, N, K);
+  return plan.slices > 1 ? plan.slices : 1;
+}
+
+// The first pass alone of a product that divides k: ws receives [slices][M][N] float32, slice z the product over the
+// z-th run of k, for a reader that adds them in their order (as the second pass of gb_gemm_bf16 would).
+extern "C" int gb_gemm_bf16_partial(const void* a, int lda, const void* w, int ldw, float* ws, long long ws_floats, int M,
+                                    int N, int K, hipStream_t stream) {
+  GB_REQUIRE(M > 16 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16_partial: bad sizes M=%d N=%d K=%d", M, N, K);
+  GB_REQUIRE(ldw % 8 == 0 && lda % 8 == 0 && lda >= K && ldw >= K, "gemm_bf16_partial: row strides (%d, %d)", lda, ldw);
+  GB_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ws && ((uintptr_t)ws % 16 == 0),
+             "gemm_bf16_partial: operands and workspace must be 16-byte aligned");
+  const SplitPlan plan = split_plan(M, N, K);
+  GB_REQUIRE(plan.slices > 1, "gemm_bf16_partial: a product of M=%d N=%d K=%d does not divide k", M, N, K);
+  GB_REQUIRE((long long)plan.floats <= ws_floats, "gemm_bf16_partial: the workspace holds %lld floats, %zu are needed", ws_floats,
+             plan.floats);
+  return launch_split<EPI_STORE, float>((const bf16*)a, lda, (const bf16*)w, ldw, (float*)nullptr, N, M, N, K, ws, plan, stream,
+                                        nullptr, 0.f, false);
+}
+
 extern "C" int gb_gemm_bf16(const void* a, int lda, const void* w, int ldw, void* c, int ldc, int c_dtype, int M, int N,
                             int K, int epilogue, const void* gamma, int gamma_dtype, float eps, const void* emit_gamma,
                             int emit_gamma_dtype, void* emit_h, int emit_ldh, float* emit_ss, const float* parts, int n_parts,
@@ -1915,6 +1940,7 @@ extern "C" int gb_gemm_bf16_rope(const void* a, int lda, const void* w, int ldw,
 
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_gemm_bf16)
+GB_TAPED(gb_gemm_bf16_partial)
 GB_TAPED(gb_gemm_bf16_grouped)
 GB_TAPED(gb_gemm_bf16_glu)
 GB_TAPED(gb_gemm_bf16_rope)

@@ -86,8 +86,8 @@ _SIGS = {
         "gb_gate_heads": [_vp, _i, _i, _vp, _i, _i, _vp, _i, _i, _i, _i, _vp],
         # z, ldz, coef, eps, out, ldo, dtype, n, d, stream
         "gb_poly_norm": [_vp, _i, _vp, _f, _vp, _i, _i, _i, _i, _vp],
-        # x, y, g, eps, rounded, dtype, n, d, stream
-        "gb_norm_add": [_vp, _vp, _vp, _f, _vp, _i, _i, _i, _vp],
+        # x, y, slices, slice stride, g, eps, rounded, dtype, n, d, conv w, taps, state, tok_seq, pos0, state slots, stream
+        "gb_norm_add": [_vp, _vp, _i, C.c_longlong, _vp, _f, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp],
     },
     "moe": {        # z, ldz, n, experts, correction, top, scale, shared, combine, ids, weights, stream
         "gb_moe_route": [_vp, _i, _i, _i, _vp, _i, _f, _i, _vp, _vp, _vp, _vp],
@@ -136,6 +136,9 @@ _SIGS = {
         # a, lda, w, ldw, c, ldc, M, N, K, limit, alpha, plus, stream
         "gb_gemm_bf16_glu": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _f, _f, _f, _vp],
         "gb_gemm_bf16_split_floats": [_i, _i, _i],
+        "gb_gemm_bf16_slices": [_i, _i, _i],
+        # a, lda, w, ldw, workspace, its floats, M, N, K, stream
+        "gb_gemm_bf16_partial": [_vp, _i, _vp, _i, _vp, C.c_longlong, _i, _i, _i, _vp],
         "gb_gemm_bf16_emit_parts": [_i, _i],
         "gb_gemm_bf16_emit_mode": [_i, _i, _i],
         # a, lda, w, ldw, c, ldc, M, N, K, gamma, gamma_dtype, eps, parts, n_parts, cos, sin, slots, k, v,
@@ -1042,19 +1045,52 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor
             _act_rows(out, z.dtype, d, "out"), dtype_code(z), n, d, _stream())
 
 
-def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, rounded: Optional[torch.Tensor] = None) -> None:
-    """x += g * y / sqrt(mean(y^2) + eps) row by row: x, y float32 [n, d], ``g`` one float32 on the device.  ``rounded``
-    ([n, d], any activations' type) receives the new x."""
+NORM_ADD_ROWS_MAX = 8192   # the widest row that headmix.hip keeps in registers (slices of y, the convolution after)
+
+
+def norm_add_takes_rows(d: int) -> bool:
+    """Whether ``norm_add`` takes y in slices, or does the next convolution, for rows of d columns."""
+    return d % 4 == 0 and d <= NORM_ADD_ROWS_MAX
+
+
+def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, rounded: Optional[torch.Tensor] = None,
+             slices: int = 1, conv: Optional[tuple] = None, ctx=None) -> None:
+    """x += g * y / sqrt(mean(y^2) + eps) row by row: x float32 [n, d], ``g`` one float32 on the device.  y is float32
+    [n, d], or with ``slices`` > 1 float32 [slices, n, d] whose sum over the slices it is (what a product that divides k
+    leaves, ``gemm_slices``).  ``rounded`` ([n, d], any activations' type) receives the new x; with ``conv=(w, state)``
+    (a step in which every request brings one row; ``ctx`` the step) it receives new x + conv(new x) instead, the rows
+    the next mixer reads, and the requests' slots in ``state`` move on as in ``time_conv``."""
     _dev(x, y, g, rounded)
     n, d = x.shape
     _f32_rows(x, (n, d), "x")
-    _f32_rows(y, (n, d), "y")
+    if slices > 1:
+        if y.dtype != torch.float32 or not y.is_contiguous() or y.numel() < slices * n * d or not norm_add_takes_rows(d):
+            raise KernelError("norm_add: slices of y must be contiguous float32 [slices, n, d], d a multiple of 4 up to "
+                              f"{NORM_ADD_ROWS_MAX}")
+    else:
+        _f32_rows(y, (n, d), "y")
     _f32_rows(g, (1,), "g")
     if rounded is not None and (tuple(rounded.shape) != (n, d) or not rounded.is_contiguous()):
         raise KernelError("norm_add: rounded must be contiguous [n, d]")
+    w = state = None
+    taps = 0
+    if conv is not None:
+        w, state = conv
+        _dev(w, state)
+        taps = w.shape[1]
+        _f32_rows(w, (d, taps), "conv w")
+        if (rounded is None or ctx is None or int(ctx.host["max_q_len"]) != 1 or not norm_add_takes_rows(d)
+                or not 1 <= taps <= TIME_CONV_MAX_TAPS):
+            raise KernelError("norm_add: the convolution after it goes with a step of single rows, a result and rows of a "
+                              f"multiple of 4 up to {NORM_ADD_ROWS_MAX} columns")
+        if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
+                         or tuple(state.shape[1:]) != (taps - 1, d)):
+            raise KernelError("norm_add: state must be contiguous float32 [slots, taps - 1, d]")
     lib = _lib("headmix")
-    _launch(lib, lib.gb_norm_add, _p(x), _p(y), _p(g), float(eps), _p(rounded),
-            dtype_code(rounded) if rounded is not None else F32, n, d, _stream())
+    _launch(lib, lib.gb_norm_add, _p(x), _p(y), int(slices), n * d, _p(g), float(eps), _p(rounded),
+            dtype_code(rounded) if rounded is not None else F32, n, d, _p(w), taps, _p(state) if taps > 1 else None,
+            _p(ctx.tok_seq) if conv is not None else None, _p(ctx.pos0) if conv is not None else None,
+            _p(ctx.state_slots) if conv is not None else None, _stream())
 
 
 # ------------------------------------------------------------------- routed experts
@@ -1254,6 +1290,29 @@ def gemm_split_floats(rows: int, n: int, k: int) -> int:
     f = _lib("gemm_bf16").gb_gemm_bf16_split_floats
     f.restype = C.c_longlong
     return int(f(int(rows), int(n), int(k)))
+
+
+def gemm_slices(rows: int, n: int, k: int) -> int:
+    """Slices into which ``gemm_partial`` divides k for a bfloat16 product of these sizes (1: it does not)."""
+    return int(_lib("gemm_bf16").gb_gemm_bf16_slices(int(rows), int(n), int(k)))
+
+
+def gemm_partial(a: torch.Tensor, w: torch.Tensor, workspace: torch.Tensor) -> int:
+    """The first pass alone of a bfloat16 product that divides k (``gemm_slices`` > 1): ``workspace`` (float32, at least
+    ``gemm_split_floats`` elements) receives [slices, rows, out features], slice z the product over the z-th run of k;
+    whoever reads them adds them in their order (``norm_add(slices=)``).  Returns the number of slices."""
+    _dev(a, w, workspace)
+    M, K = a.shape
+    N = w.shape[0]
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != K:
+        raise KernelError(f"gemm_partial: bfloat16 operands of one inner size, got a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}")
+    if workspace.dtype != torch.float32 or not workspace.is_contiguous():
+        raise KernelError("gemm_partial: the workspace must be contiguous float32")
+    slices = gemm_slices(M, N, K)
+    lib = _lib("gemm_bf16")
+    _launch(lib, lib.gb_gemm_bf16_partial, _p(a), _rows(a, "a"), _p(w), _rows(w, "w"), _p(workspace), workspace.numel(), M, N, K,
+            _stream())
+    return slices
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, silu_mul: bool = False,

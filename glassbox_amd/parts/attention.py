@@ -16,7 +16,7 @@ import torch
 
 from .. import ops
 from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, StateSpec, TensorSpec, emit_target,
-                   needs_multiple_of_8, product, split_workspace)
+                   needs_multiple_of_8, product, product_in_slices, split_workspace)
 
 
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, n_heads: int, scale: float,
@@ -207,7 +207,8 @@ class TiedValueAttention(Mixer):
         return out
 
     def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
-        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        """Adds the mixed rows into ``residual``; with ``store`` writes them there instead (float32 either way) or leaves
+        them in slices, and returns what ``product_in_slices`` does."""
         if cache is None or cache.k_pages is None:
             raise ValueError("TiedValueAttention needs a layer cache with pages")
         n = h.shape[0]
@@ -312,7 +313,8 @@ class ShortConvAttention(Mixer):
         return out
 
     def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
-        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        """Adds the mixed rows into ``residual``; with ``store`` writes them there instead (float32 either way) or leaves
+        them in slices, and returns what ``product_in_slices`` does."""
         if cache is None or cache.k_pages is None or (self.taps > 1 and cache.state is None):
             raise ValueError("ShortConvAttention needs a layer cache with pages (and state, with a convolution)")
         n = h.shape[0]
@@ -399,7 +401,8 @@ class LatentAttention(Mixer):
         return []
 
     def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
-        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        """Adds the mixed rows into ``residual``; with ``store`` writes them there instead (float32 either way) or leaves
+        them in slices, and returns what ``product_in_slices`` does."""
         if cache is None or cache.k_pages is None:
             raise ValueError("LatentAttention needs a layer cache with pages")
         n = h.shape[0]
@@ -428,7 +431,10 @@ class LatentAttention(Mixer):
         paged_attention(ctx, heads[:, :H * hc], att, cache, H, self.scale, self.window)
         gated = ctx.buffer("latent_gated", (n, H * V), ctx.dtype)
         ops.gate_heads(att, hc, first[:, shared + R:shared + R + H * V], gated, H, V)
-        product(ctx, gated, self.wo, residual, accumulate=not store)
+        if store:   # the caller's norm adds the slices of a product that divides k
+            return product_in_slices(ctx, gated, self.wo, residual)
+        product(ctx, gated, self.wo, residual, accumulate=True)
+        return None
 
 
 class DifferentialAttention(Mixer):
@@ -485,7 +491,8 @@ class DifferentialAttention(Mixer):
         return []
 
     def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
-        """Adds the mixed rows into ``residual``, or with ``store`` writes them there (float32 either way)."""
+        """Adds the mixed rows into ``residual``; with ``store`` writes them there instead (float32 either way) or leaves
+        them in slices, and returns what ``product_in_slices`` does."""
         if cache is None or cache.k_pages is None:
             raise ValueError("DifferentialAttention needs a layer cache with pages")
         n = h.shape[0]
@@ -504,4 +511,7 @@ class DifferentialAttention(Mixer):
         paged_attention(ctx, heads[:, :2 * H * hc], att, cache, 2 * H, self.scale, 0)
         o = ctx.buffer("diff_o", (n, H * V), ctx.dtype)
         ops.diff_combine(att, hc, self.lam, 1.0 - self.diff, self.eps, o, H, V)
-        product(ctx, o, self.wo, residual, accumulate=not store)
+        if store:   # the caller's norm adds the slices of a product that divides k
+            return product_in_slices(ctx, o, self.wo, residual)
+        product(ctx, o, self.wo, residual, accumulate=True)
+        return None

@@ -253,6 +253,23 @@ def product(ctx, a, w, out, accumulate: bool = False) -> None:
         ops.gemm_plain(a, w, out, accumulate=accumulate)
 
 
+def product_in_slices(ctx, a, w, out):
+    """``out = a . w^T`` for a caller whose next pass reads the rows once and can add them up on the way
+    (``ScalarRMSNorm.add_normed``): where the product divides k over workgroups only its first pass runs, and
+    ``(workspace, slices)`` comes back in place of ``(out, 1)``; the slices are [slices, rows, out features]."""
+    from .. import ops
+    n, k = a.shape
+    width = w.shape[0]
+    if ops.gemm_takes(a, w) and ops.norm_add_takes_rows(width) and ctx.dtype == torch.bfloat16 and n > 16:
+        slices = ops.gemm_slices(n, width, k)
+        ws = split_workspace(ctx, n, width, k) if slices > 1 else None
+        if ws is not None and ws.numel() >= slices * n * width:
+            ops.gemm_partial(a, w, ws)
+            return ws, slices
+    product(ctx, a, w, out)
+    return out, 1
+
+
 class Mixer(Part):
     cache_spec: Optional[CacheSpec] = None
     state_spec: Optional[StateSpec] = None

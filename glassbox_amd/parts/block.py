@@ -165,20 +165,30 @@ class OutputNormBlock(Block):
     def state_spec(self) -> Optional[StateSpec]:
         return self.conv.state_spec if self.conv.state_spec is not None else self.mixer.state_spec
 
-    def forward(self, ctx, x, cache: Optional[LayerCache]):
+    def entry_rows(self, ctx, n: int, cache: Optional[LayerCache]):
+        """``(weight, state)`` of the convolution this block begins with, if the pass that makes the residual before
+        it may also make the rows this block's mixer reads (``forward(..., pre=)`` then takes them): a step of
+        single tokens, whose rows need nothing of the step's other rows; else None."""
+        return self.conv.entry_spec(ctx, n, cache) if hasattr(self.conv, "entry_spec") else None
+
+    def forward(self, ctx, x, cache: Optional[LayerCache], pre=None, emit=None):
+        """``pre``: the rows this block's mixer reads, made by the block before; ``emit``: the ``entry_rows`` of the block
+        after.  Returns the rows for that block if the last norm's pass made them."""
         n, width = x.shape
-        h = self.conv.forward(ctx, x, cache)
+        h = pre if pre is not None else self.conv.forward(ctx, x, cache)
         y = ctx.buffer("sublayer_y", (n, width), torch.float32)
-        self.mixer.forward(ctx, h, y, cache, store=True)
+        # a sublayer's rows lie in y, or in slices that the norm's pass adds up (``product_in_slices``)
+        made, slices = self.mixer.forward(ctx, h, y, cache, store=True) or (y, 1)
+        handed = ctx.buffer("h", (n, width), ctx.dtype) if emit is not None else None
         if self.ffn is None:
-            self.mixer_norm.add_normed(ctx, y, x)
-            return None
+            self.mixer_norm.add_normed(ctx, made, x, rounded=handed, slices=slices, conv=emit)
+            return handed
         if ctx.dtype == torch.float32:
-            self.mixer_norm.add_normed(ctx, y, x)
+            self.mixer_norm.add_normed(ctx, made, x, slices=slices)
             rows = x
         else:   # the pass that makes the residual also leaves it in the activations' type for the feed-forward
             rows = ctx.buffer("h", (n, width), ctx.dtype)
-            self.mixer_norm.add_normed(ctx, y, x, rounded=rows)
-        self.ffn.forward(ctx, rows, y, store=True)
-        self.ffn_norm.add_normed(ctx, y, x)
-        return None
+            self.mixer_norm.add_normed(ctx, made, x, rounded=rows, slices=slices)
+        made, slices = self.ffn.forward(ctx, rows, y, store=True) or (y, 1)
+        self.ffn_norm.add_normed(ctx, made, x, rounded=handed, slices=slices, conv=emit)
+        return handed

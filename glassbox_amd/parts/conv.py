@@ -33,6 +33,14 @@ class TimeConv(Part):
             return [("taps", f"{self.taps} is above {ops.TIME_CONV_MAX_TAPS}, the longest convolution the kernel takes")]
         return []
 
+    def entry_spec(self, ctx, n: int, cache: Optional[LayerCache]):
+        """``(weight, state)`` for ``ops.norm_add(conv=)`` if the pass that adds a normed sublayer into the residual may
+        make this convolution's rows as well (every request of the step brings one row), else None."""
+        if (not self.taps or int(ctx.host["max_q_len"]) != 1 or not ops.norm_add_takes_rows(self.width)
+                or (self.taps > 1 and (cache is None or cache.state is None))):
+            return None
+        return (self.weight, cache.state if self.taps > 1 else None)
+
     def forward(self, ctx, x, cache: Optional[LayerCache], out_name: str = "h") -> torch.Tensor:
         """The rows a mixer reads, in the activations' type; moves the requests' state on (call it before x changes)."""
         if self.taps > 1 and (cache is None or cache.state is None):

@@ -7,7 +7,8 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import FeedForward, PreNormed, TensorSpec, emit_target, needs_multiple_of_8, product, split_workspace
+from .base import (FeedForward, PreNormed, TensorSpec, emit_target, needs_multiple_of_8, product, product_in_slices,
+                   split_workspace)
 
 
 class SwiGLU(FeedForward):
@@ -111,7 +112,9 @@ class ClampedGLU(FeedForward):
             gate_up = ctx.buffer("glu_gate_up", (n, 2 * self.intermediate), torch.float32)
             product(ctx, h, self.w_gate_up, gate_up)
             ops.glu_clamped(gate_up, act, self.limit, self.alpha)
-        product(ctx, act, self.w_down, residual, accumulate=not store)
+        if store:   # the caller's norm adds the slices of a product that divides k
+            return product_in_slices(ctx, act, self.w_down, residual)
+        product(ctx, act, self.w_down, residual, accumulate=True)
         return None
 
 
@@ -144,5 +147,7 @@ class PolyNormMLP(FeedForward):
         product(ctx, h, self.w_up, z)
         act = ctx.buffer("act", (n, self.intermediate), ctx.dtype)
         ops.poly_norm(z, self.coef, self.eps, act)
-        product(ctx, act, self.w_down, residual, accumulate=not store)
+        if store:   # the caller's norm adds the slices of a product that divides k
+            return product_in_slices(ctx, act, self.w_down, residual)
+        product(ctx, act, self.w_down, residual, accumulate=True)
         return None

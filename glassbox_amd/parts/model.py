@@ -146,7 +146,7 @@ class DecoderModel(Part):
             self.embedding.forward(ctx, x)
         if keep:
             x, embedded = x[0], x[1]
-        pre = None   # what the block before prepared of this block's first norm
+        pre = pre_kind = None   # what the block before prepared of this block's first norm (or of the rows it reads)
         if self._taped is None:
             self._taped = [b.all_taped() for b in self.blocks]
         tapes = None
@@ -163,16 +163,23 @@ class DecoderModel(Part):
             block = self.blocks[call.block]
             if call.enter is not None:
                 self.passes.forward(ctx, x, embedded, call.enter)
-                pre = None   # (what the block before prepared was of the residual before this)
-            handover = hasattr(block, "entry_norm")
+                pre = pre_kind = None   # (what the block before prepared was of the residual before this)
+            # what a block hands to the next: the work of that block's first norm (entry_norm), or the rows its mixer
+            # reads (entry_rows, which also needs the cache layer that holds the next block's state)
+            handover = "entry_norm" if hasattr(block, "entry_norm") else "entry_rows" if hasattr(block, "entry_rows") else None
             more = {}
             if handover:
                 last = i + 1 == len(self.schedule)
                 after = None if last else self.blocks[self.schedule[i + 1].block]
                 if not last and self.schedule[i + 1].enter is not None:
                     after = None   # the residual changes before the next block reads it: nothing to prepare
-                more = {"pre": pre, "emit": after.entry_norm(ctx, ctx.n) if hasattr(after, "entry_norm") else None}
-                if last and self._head_takes_prepared(ctx):
+                more = {"pre": pre if pre_kind == handover else None, "emit": None}
+                if handover == "entry_norm" and hasattr(after, "entry_norm"):
+                    more["emit"] = after.entry_norm(ctx, ctx.n)
+                elif handover == "entry_rows" and hasattr(after, "entry_rows"):
+                    nxt = self.schedule[i + 1]
+                    more["emit"] = after.entry_rows(ctx, ctx.n, caches[nxt.cache] if nxt.cache is not None else None)
+                if handover == "entry_norm" and last and self._head_takes_prepared(ctx):
                     # the last block prepares the final norm as it would the next block's first
                     more["emit"] = self.final_norm.emit_spec(ctx, ctx.n)
             if tapes is not None and self._taped[call.block]:
@@ -180,7 +187,7 @@ class DecoderModel(Part):
                 out = tapes.forward(i, block, x, cache, more)
             else:
                 out = block.forward(ctx, x, cache, **more)
-            pre = out if handover else None
+            pre, pre_kind = (out, handover) if handover else (None, None)
         if ctx.want.numel() == 0:
             return ctx.buffer("logits", (0, self.vocab_size), torch.float32)
         if self._head_takes_prepared(ctx) and isinstance(pre, (PreNormed, Normed)):

@@ -78,6 +78,7 @@ class ScalarRMSNorm(Norm):
         ops.rmsnorm(x, self.weight, self.eps, out, rows)
         return out
 
-    def add_normed(self, ctx, y, x, rounded=None) -> None:
-        """x += g * y / sqrt(mean(y^2) + eps) (both float32); ``rounded`` receives the new x in its own type."""
-        ops.norm_add(x, y, self.gain, self.eps, rounded)
+    def add_normed(self, ctx, y, x, rounded=None, slices: int = 1, conv=None) -> None:
+        """x += g * y / sqrt(mean(y^2) + eps) (both float32; ``slices`` > 1: y is the sum of that many pieces);
+        ``rounded`` receives the new x in its own type, or with ``conv=(weight, state)`` what a ``TimeConv`` makes of it."""
+        ops.norm_add(x, y, self.gain, self.eps, rounded, slices=slices, conv=conv, ctx=ctx)

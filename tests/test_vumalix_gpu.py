@@ -118,6 +118,99 @@ def test_norms_of_slices_the_polynomial_the_gate_and_the_normed_add(dtype):
         assert (xd.cpu().to(F64) - want - pv.scalar_norm(y, g, 1e-5)).abs().max() < 4e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rows_in_registers_many_rows_and_few(dtype):
+    """The polynomial and the normed add keep a row in registers, with other threads a row for many rows than for few."""
+    from glassbox_amd import ops
+    torch.manual_seed(21)
+    f = lambda t: t.to(dtype).to(F64)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    for n, ff in ((3, 1536), (700, 264), (520, 8200)):
+        z = f(torch.randn(n, ff, dtype=F64) * 1.5)
+        coef = torch.tensor([0.5, 0.4, -0.2, 0.3]).to(F64)
+        out = torch.empty(n, ff + 8, dtype=dtype, device=DEV)[:, :ff]
+        ops.poly_norm(_dev(z, dtype), _dev(coef), 1e-5, out)
+        want = pv.poly_norm(z, coef, 1e-5)
+        assert (out.cpu().to(F64) - want).abs().max() < tol * float(want.abs().max())
+    for n, d in ((600, 72), (513, 4100)):
+        x, y, g = torch.randn(n, d).to(F64), (torch.randn(n, d) * 3).to(F64), torch.tensor([0.8]).to(F64)
+        xd, r = _dev(x), torch.empty(n, d, dtype=dtype, device=DEV)
+        ops.norm_add(xd, _dev(y), _dev(g), 1e-5, r)
+        want = x + pv.scalar_norm(y, g, 1e-5)
+        assert (xd.cpu().to(F64) - want).abs().max() < 4e-6 and (r.cpu().to(F64) - want).abs().max() < tol * 2
+
+
+def test_a_product_left_in_slices_and_the_normed_add_that_adds_them():
+    """``gemm_partial`` leaves the sums over the runs of k side by side; their sum is the product, and ``norm_add`` with
+    ``slices`` gives what it gives of the whole product."""
+    from glassbox_amd import ops
+    torch.manual_seed(4)
+    for n, width, k in ((40, 64, 2048), (600, 128, 8192)):
+        slices = ops.gemm_slices(n, width, k)
+        assert slices > 1 and ops.gemm_split_floats(n, width, k) >= slices * n * width
+        a, w = (torch.randn(n, k) * 0.5).to(torch.bfloat16), (torch.randn(width, k) * 0.1).to(torch.bfloat16)
+        ws = torch.full((ops.gemm_split_floats(n, width, k) + 16,), 7.0, device=DEV)
+        assert ops.gemm_partial(a.to(DEV), w.to(DEV), ws) == slices
+        whole = torch.empty(n, width, device=DEV)
+        ops.gemm(a.to(DEV), w.to(DEV), whole, workspace=torch.empty_like(ws))
+        parts = ws[:slices * n * width].view(slices, n, width)
+        assert (parts.to(F64).sum(0) - whole.to(F64)).abs().max() < 1e-4
+        assert (whole.cpu().to(F64) - a.to(F64) @ w.to(F64).T).abs().max() < 2e-3
+        assert torch.all(ws[slices * n * width:] == 7.0)
+        x, g = torch.randn(n, width).to(F64), torch.tensor([1.7]).to(F64)
+        one, two = _dev(x), _dev(x)
+        r1, r2 = (torch.empty(n, width, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+        ops.norm_add(one, whole, _dev(g), 1e-5, r1)
+        ops.norm_add(two, ws, _dev(g), 1e-5, r2, slices=slices)
+        assert torch.equal(one, two) and torch.equal(r1, r2)
+        assert (one.cpu().to(F64) - x - pv.scalar_norm(whole.cpu().to(F64), g, 1e-5)).abs().max() < 4e-6
+
+
+@pytest.mark.parametrize("d, taps, dtype", [(64, 4, torch.float32), (96, 5, torch.bfloat16), (24, 2, torch.bfloat16), (16, 1, torch.float32)])
+def test_the_normed_add_that_makes_the_next_convolutions_rows(d, taps, dtype):
+    """Steps of single tokens: the pass that adds a normed sublayer into the residual also writes x + conv(x) of the new
+    residual and moves the slots on.  One request begins in a portion that ``time_conv`` takes, the other at its first
+    token in a slot that holds garbage; a third joins later."""
+    from glassbox_amd import ops
+    torch.manual_seed(d * taps)
+    K = taps - 1
+    lens = {0: 12, 1: 7, 2: 4}
+    begin = {0: 0, 1: 0, 2: 3}            # the step in which a request begins (request 0 with a portion of 5)
+    slots = {0: 3, 1: 1, 2: 0}
+    w = torch.randn(d, taps).float()
+    g = torch.tensor([0.7])
+    state = torch.full((5, max(K, 1), d), 55.0, device=DEV) if K else None
+    xs = {r: torch.randn(T, d).float() for r, T in lens.items()}           # the residual before the sublayer's rows are added
+    ys = {r: (torch.randn(T, d) * 4).float() for r, T in lens.items()}
+    new = {r: xs[r].to(F64) + pv.scalar_norm(ys[r].to(F64), g.to(F64), 1e-5) for r in lens}
+    want = {r: pv.mixer_input(new[r], w.to(F64)) for r in lens}
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    # request 0's first five rows in one portion: the residual as it is after the add, through the convolution's own kernel
+    ctx = _step_ctx([(0, 0, 5)], slots)
+    out = torch.empty(5, d, dtype=dtype, device=DEV)
+    ops.time_conv(_dev(new[0][:5]), _dev(w), state, ctx, out)
+    assert (out.cpu().to(F64) - want[0][:5]).abs().max() < tol * float(want[0].abs().max())
+    done = {0: 5, 1: 0, 2: 0}
+    for step in range(8):
+        rows = [(r, done[r], done[r] + 1) for r in lens if step >= begin[r] and done[r] < lens[r]]
+        if not rows:
+            break
+        ctx = _step_ctx(rows, slots)
+        x = _dev(torch.stack([xs[r][a] for r, a, _ in rows]))
+        y = _dev(torch.stack([ys[r][a] for r, a, _ in rows]))
+        out = torch.empty(len(rows), d, dtype=dtype, device=DEV)
+        ops.norm_add(x, y, _dev(g), 1e-5, out, conv=(_dev(w), state), ctx=ctx)
+        for i, (r, a, b) in enumerate(rows):
+            assert (x[i].cpu().to(F64) - new[r][a]).abs().max() < 4e-6
+            assert (out[i].cpu().to(F64) - want[r][a]).abs().max() < tol * float(want[r].abs().max()), (step, r)
+            done[r] = b
+            if K:
+                kept = state[slots[r]].cpu().to(F64)
+                assert all((kept[i2] - new[r][b - K + i2]).abs().max() < 4e-6 for i2 in range(K) if b - K + i2 >= 0)
+    if K:
+        assert torch.all(state[2] == 55.0) and torch.all(state[4] == 55.0)
+
+
 # ------------------------------------------------------------------------------------------ heads and their attention
 def _pool(T, P, G, hc, dtype):
     from glassbox_amd import ops
