@@ -1,7 +1,7 @@
 // What stands around the attention of two mixers and around sublayers whose *output* is normed:
 //
 //   time_conv      h = x + conv(x): a short causal convolution over time on every channel of the 32-bit residual,
-//                  conv(x)[t, c] = sum_j w[c, j] x[t - taps + 1 + j, c], zeros before the request's first token.  The last
+//                  conv(x)[t, c] = sum_j w[j, c] x[t - taps + 1 + j, c] (the weights a row a tap), zeros before the request's first token.  The last
 //                  taps - 1 rows of x of each request live in its state slot, [taps - 1, channels] float32 (index i is the
 //                  position `first position of the step` - (taps - 1) + i).
 //   norm_slices    RMS norms with a weight over one or two runs of columns of a row (the latents of queries and of
@@ -114,7 +114,7 @@ __global__ void time_conv_kernel(const float* __restrict__ x, int ldx, const flo
     } else if (first_pos + off - back >= 0) {
       v = st[(size_t)(off + j) * d];   // index (position - back) - first_pos + K
     }
-    acc = fmaf(w[(size_t)c * taps + j], v, acc);
+    acc = fmaf(w[(size_t)j * d + c], v, acc);
   }
   out[(size_t)t * ldo + c] = from_f<T>(cur + acc);
   if (single) {
@@ -135,36 +135,48 @@ __global__ __launch_bounds__(256) void time_conv4_kernel(const float* __restrict
                                                          int d, int single) {
   const int t = blockIdx.x, c = (blockIdx.y * 256 + threadIdx.x) * 4;
   if (c >= d) return;
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   const f32x4 cur = *reinterpret_cast<const f32x4*>(x + (size_t)t * ldx + c);
   if (taps <= 0) {
     store4(out + (size_t)t * ldo + c, cur);
     return;
   }
   const int K = taps - 1;
+  // the rows before this one and the weights are asked for before the request's tables say which of the rows count:
+  // the loads of a token are then all on their way together
+  f32x4 rows[kMaxTaps - 1];
+  f32x4 wv[kMaxTaps];
+#pragma unroll
+  for (int j = 0; j < kMaxTaps - 1; ++j) {
+    const int back = K - j;
+    rows[j] = (j < K && !single && t - back >= 0) ? *reinterpret_cast<const f32x4*>(x + (size_t)(t - back) * ldx + c) : zero;
+  }
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) wv[j] = j < taps ? *reinterpret_cast<const f32x4*>(w + (size_t)j * d + c) : zero;
   const int seq = tok_seq[t], off = t - q_start[seq], first_pos = pos0[seq];
   float* st = K > 0 ? state + (size_t)state_slots[seq] * K * d + c : nullptr;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   f32x4 old[kMaxTaps - 1];
   if (single) {
 #pragma unroll
     for (int i = 0; i < kMaxTaps - 1; ++i)
       if (i < K) old[i] = *reinterpret_cast<const f32x4*>(st + (size_t)i * d);
   }
+  f32x4 acc = zero;
 #pragma unroll
   for (int j = 0; j < kMaxTaps; ++j) {
     if (j >= taps) break;
     const int back = K - j;   // how many tokens before this one
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    f32x4 v = zero;
     if (back == 0) {
       v = cur;
     } else if (off >= back) {
-      v = *reinterpret_cast<const f32x4*>(x + (size_t)(t - back) * ldx + c);
+      v = rows[j < kMaxTaps - 1 ? j : 0];
     } else if (first_pos + off - back >= 0) {
       // index (position - back) - first_pos + K of the slot; a step of single tokens has off = 0 and the slot in hand
       v = single ? old[j < kMaxTaps - 1 ? j : 0] : *reinterpret_cast<const f32x4*>(st + (size_t)(off + j) * d);
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[e] = fmaf(w[(size_t)(c + e) * taps + j], v[e], acc[e]);
+    for (int e = 0; e < 4; ++e) acc[e] = fmaf(wv[j][e], v[e], acc[e]);
   }
   store4(out + (size_t)t * ldo + c, cur + acc);
   if (single) {
@@ -636,8 +648,9 @@ __global__ __launch_bounds__(THREADS) void norm_add_rows_kernel(float* __restric
             if (j > 0) *reinterpret_cast<f32x4*>(st + (size_t)(j - 1) * d + c) = in;
             if (pos - (K - j) < 0) in = f32x4{0.f, 0.f, 0.f, 0.f};   // before the request's first token
           }
+          const f32x4 wj = *reinterpret_cast<const f32x4*>(conv_w + (size_t)j * d + c);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[e] = fmaf(conv_w[(size_t)(c + e) * taps + j], in[e], acc[e]);
+          for (int e = 0; e < 4; ++e) acc[e] = fmaf(wj[e], in[e], acc[e]);
         }
         if (K > 0) *reinterpret_cast<f32x4*>(st + (size_t)(K - 1) * d + c) = nx;
         store4(rounded + (size_t)t * d + c, nx + acc);
@@ -663,7 +676,7 @@ inline bool grid_fits(long long count, int per_block) { return (count + per_bloc
     return fail(what ": unknown dtype %d", dtype);  \
   }
 
-// x [n, ldx] float32, w [d, taps] float32 (taps 0: none, out = x rounded), state [slots, taps - 1, d] float32,
+// x [n, ldx] float32, w [taps, d] float32 (taps 0: none, out = x rounded), state [slots, taps - 1, d] float32,
 // out [n, ldo] of `dtype`.  single: every request brings one row and its slot is moved on here; otherwise the caller moves
 // the slots after this call, before x changes.
 extern "C" int gb_time_conv(const float* x, int ldx, const float* w, int taps, float* state, const int32_t* tok_seq,
@@ -676,7 +689,7 @@ extern "C" int gb_time_conv(const float* x, int ldx, const float* w, int taps, f
   if (n == 0) return 0;
   const long long count = (long long)n * d;
   GB_REQUIRE(grid_fits(count, 256), "time_conv: too many elements");
-  if (d % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && words16(x) && words16(out) && words16(state) && (d + 1023) / 1024 < 65536) {
+  if (d % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && words16(x) && words16(out) && words16(state) && words16(w) && (d + 1023) / 1024 < 65536) {
     const dim3 grid4((unsigned)n, (unsigned)((d + 1023) / 1024));
     GB_BY_DTYPE(dtype, "time_conv",
                 hipLaunchKernelGGL(time_conv4_kernel<TT>, grid4, dim3(256), 0, stream, x, ldx, w, taps, state, tok_seq, q_start,
@@ -850,7 +863,7 @@ extern "C" int gb_poly_norm(const void* z, int ldz, const float* coef, float eps
 }
 
 // x, y [n, d] float32, g one float32 on the device; rounded (or nullptr) [n, d] of `dtype` receives the new x.
-// slices > 1: y is the sum of that many [n, d] pieces, slice_stride floats apart.  conv_w (float32 [d, taps]; a step in
+// slices > 1: y is the sum of that many [n, d] pieces, slice_stride floats apart.  conv_w (float32 [taps, d]; a step in
 // which every request brings one row): rounded receives x + conv(x) of the new x, and the requests' slots in
 // state [slots, taps - 1, d] are moved on by this row.
 extern "C" int gb_norm_add(float* x, const float* y, int slices, long long slice_stride, const float* g, float eps,
@@ -861,7 +874,7 @@ extern "C" int gb_norm_add(float* x, const float* y, int slices, long long slice
   GB_REQUIRE(!conv_w || (rounded && taps >= 1 && taps <= kMaxTaps && tok_seq && pos0 && state_slots && (taps == 1 || state)),
              "norm_add: the convolution needs a result, weights of at most %d taps, the step's tables and the state", kMaxTaps);
   if (n == 0) return 0;
-  const bool words = d % 4 == 0 && d <= 8192 && words16(x) && words16(y) && words16(rounded) && words16(state) &&
+  const bool words = d % 4 == 0 && d <= 8192 && words16(x) && words16(y) && words16(rounded) && words16(state) && words16(conv_w) &&
                      slice_stride % 4 == 0;
   GB_REQUIRE(words || (slices == 1 && !conv_w), "norm_add: slices and the convolution take rows of at most 8192 columns, a multiple of 4");
   if (words) {

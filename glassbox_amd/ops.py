@@ -898,8 +898,8 @@ def _act_rows(t: torch.Tensor, dtype, cols: int, what: str) -> int:
 
 
 def time_conv(x: torch.Tensor, w: Optional[torch.Tensor], state: Optional[torch.Tensor], ctx, out: torch.Tensor) -> None:
-    """out = x + conv(x) in the type of ``out``: x float32 [n, d] (the residual), ``w`` float32 [d, taps] (None: out is x
-    rounded), conv(x)[t] = sum_j w[:, j] x[t - taps + 1 + j] over the request's own tokens, zeros before its first.  The
+    """out = x + conv(x) in the type of ``out``: x float32 [n, d] (the residual), ``w`` float32 [taps, d], a row a tap (None: out is x
+    rounded), conv(x)[t] = sum_j w[j] x[t - taps + 1 + j] over the request's own tokens, zeros before its first.  The
     request's last taps - 1 rows of x live in ``state`` (float32 [slots, taps - 1, d]) and are moved on by this call, so
     it must come before x changes."""
     _dev(x, w, state, out)
@@ -907,8 +907,8 @@ def time_conv(x: torch.Tensor, w: Optional[torch.Tensor], state: Optional[torch.
     _f32_rows(x, (n, d), "x")
     taps = 0
     if w is not None:
-        taps = w.shape[1]
-        _f32_rows(w, (d, taps), "w")
+        taps = w.shape[0]
+        _f32_rows(w, (taps, d), "w")
         if taps > TIME_CONV_MAX_TAPS:
             raise KernelError(f"time_conv: {taps} taps are above {TIME_CONV_MAX_TAPS}")
         if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
@@ -1057,7 +1057,7 @@ def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, roun
              slices: int = 1, conv: Optional[tuple] = None, ctx=None) -> None:
     """x += g * y / sqrt(mean(y^2) + eps) row by row: x float32 [n, d], ``g`` one float32 on the device.  y is float32
     [n, d], or with ``slices`` > 1 float32 [slices, n, d] whose sum over the slices it is (what a product that divides k
-    leaves, ``gemm_slices``).  ``rounded`` ([n, d], any activations' type) receives the new x; with ``conv=(w, state)``
+    leaves, ``gemm_slices``).  ``rounded`` ([n, d], any activations' type) receives the new x; with ``conv=(w, state)``, w [taps, d] as ``time_conv`` takes it
     (a step in which every request brings one row; ``ctx`` the step) it receives new x + conv(new x) instead, the rows
     the next mixer reads, and the requests' slots in ``state`` move on as in ``time_conv``."""
     _dev(x, y, g, rounded)
@@ -1077,8 +1077,8 @@ def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, roun
     if conv is not None:
         w, state = conv
         _dev(w, state)
-        taps = w.shape[1]
-        _f32_rows(w, (d, taps), "conv w")
+        taps = w.shape[0]
+        _f32_rows(w, (taps, d), "conv w")
         if (rounded is None or ctx is None or int(ctx.host["max_q_len"]) != 1 or not norm_add_takes_rows(d)
                 or not 1 <= taps <= TIME_CONV_MAX_TAPS):
             raise KernelError("norm_add: the convolution after it goes with a step of single rows, a result and rows of a "

@@ -26,7 +26,7 @@ class TimeConv(Part):
 
     def load(self, tensors):
         if self.taps:
-            self.weight = tensors["weight"].float().contiguous()
+            self.weight = tensors["weight"].float().t().contiguous()   # a row a tap: neighbouring channels side by side
 
     def problems(self, dtype, page_size):
         if self.taps > ops.TIME_CONV_MAX_TAPS:

@@ -64,7 +64,7 @@ def test_the_convolution_of_the_residual_in_portions(d, taps, dtype):
         n = sum(b - a for _, a, b in rows)
         x = _dev(torch.cat([data[r][a:b] for r, a, b in rows], 0))
         out = torch.full((n, d + 3), 9.0, dtype=dtype, device=DEV)[:, :d]   # rows wider than the residual
-        ops.time_conv(x, _dev(w) if taps else None, state, ctx, out)
+        ops.time_conv(x, _dev(w.t()) if taps else None, state, ctx, out)
         got, at = out.cpu().to(F64), 0
         for r, a, b in rows:
             assert (got[at:at + b - a] - want[r][a:b]).abs().max() < tol * max(1.0, float(want[r].abs().max())), (step, r)
@@ -188,7 +188,7 @@ def test_the_normed_add_that_makes_the_next_convolutions_rows(d, taps, dtype):
     # request 0's first five rows in one portion: the residual as it is after the add, through the convolution's own kernel
     ctx = _step_ctx([(0, 0, 5)], slots)
     out = torch.empty(5, d, dtype=dtype, device=DEV)
-    ops.time_conv(_dev(new[0][:5]), _dev(w), state, ctx, out)
+    ops.time_conv(_dev(new[0][:5]), _dev(w.t()), state, ctx, out)
     assert (out.cpu().to(F64) - want[0][:5]).abs().max() < tol * float(want[0].abs().max())
     done = {0: 5, 1: 0, 2: 0}
     for step in range(8):
@@ -199,7 +199,7 @@ def test_the_normed_add_that_makes_the_next_convolutions_rows(d, taps, dtype):
         x = _dev(torch.stack([xs[r][a] for r, a, _ in rows]))
         y = _dev(torch.stack([ys[r][a] for r, a, _ in rows]))
         out = torch.empty(len(rows), d, dtype=dtype, device=DEV)
-        ops.norm_add(x, y, _dev(g), 1e-5, out, conv=(_dev(w), state), ctx=ctx)
+        ops.norm_add(x, y, _dev(g), 1e-5, out, conv=(_dev(w.t()), state), ctx=ctx)
         for i, (r, a, b) in enumerate(rows):
             assert (x[i].cpu().to(F64) - new[r][a]).abs().max() < 4e-6
             assert (out[i].cpu().to(F64) - want[r][a]).abs().max() < tol * float(want[r].abs().max()), (step, r)
