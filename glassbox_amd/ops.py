@@ -1557,22 +1557,18 @@ def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int, k
 
 
 @functools.lru_cache(maxsize=4096)   # a pure function of the sizes, asked for at every product
-def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int, window: int = 0) -> int:
+def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
     """Keys per workgroup of the decode kernel: a multiple of 256.  With a workgroup for every compute
     unit from requests and kv heads alone (or for half of them, if the context is short), each takes a whole
     context (and sixteen waves: nothing is left to combine afterwards); otherwise small enough that the launch
-    has about a thousand workgroups with keys.  Under a ``window`` (without kept first keys) only the chunks that
-    the window touches have keys, so it is the window's keys that are divided."""
+    has about a thousand workgroups."""
     groups = max(1, n_decode * n_kv_heads)
-    live = min(max_context, window) if window > 0 else max_context      # keys a request reads
     want_splits = 1 if groups >= 256 else min(256, max(1, 1024 // groups))   # the second pass combines up to 256
-    if groups >= 128 and live <= 1024:
+    if groups >= 128 and max_context <= 1024:
         # sixteen waves take a thousand keys in one round: the second pass would cost more than it saves (measured:
         # 32 requests of SmolLM2-360M -6 % a step, 4 of SmolLM2-1.7B -2 %; with 64 workgroups or 2,048 keys it is slower)
         want_splits = 1
-    if want_splits == 1:
-        return max(256, -(-max_context // 256) * 256)
-    chunk = max(-(-live // want_splits), -(-max_context // 256))        # at most 256 chunks in all
+    chunk = -(-max_context // want_splits)
     return max(256, -(-chunk // 256) * 256)
 
 
@@ -1587,7 +1583,7 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
         raise KernelError("attention_decode: q and out must be bfloat16 [n, heads * head size]")
     tables = ctx.tables[cache.group]
     max_context = int(ctx.host["max_context"])
-    chunk = decode_chunk(n_dec, nkv, max_context, 0 if keep_first else window)
+    chunk = decode_chunk(n_dec, nkv, max_context)
     splits = -(-max_context // chunk)
     ws_acc = ctx.buffer("attn_ws_acc", (n_dec * n_heads * splits * hd,), torch.float32)
     ws_ml = ctx.buffer("attn_ws_ml", (n_dec * n_heads * splits * 2,), torch.float32)
