@@ -186,6 +186,61 @@ __global__ __launch_bounds__(256) void time_conv4_kernel(const float* __restrict
   }
 }
 
+// Steps with portions: four channels and four tokens in a row a thread, so that a row of x is read for four tokens'
+// sums and not for one (taps + 3 rows where four tokens alone would read 4 taps).  The tokens may be of different
+// requests; each looks up its own.
+constexpr int kConvTokens = 4;
+template <typename T>
+__global__ __launch_bounds__(256) void time_conv4x4_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                           int taps, const float* __restrict__ state,
+                                                           const int32_t* __restrict__ tok_seq,
+                                                           const int32_t* __restrict__ q_start,
+                                                           const int32_t* __restrict__ pos0,
+                                                           const int32_t* __restrict__ state_slots, T* __restrict__ out,
+                                                           int ldo, int n, int d) {
+  const int t0 = blockIdx.x * kConvTokens, c = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c >= d) return;
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+  const int K = taps - 1;
+  // rows[k] is the row of token t0 - K + k: what the four tokens' taps can reach of the step's rows; tap j of token
+  // t0 + i reads rows[i + j]
+  f32x4 rows[kMaxTaps - 1 + kConvTokens], cur[kConvTokens], wv[kMaxTaps];
+#pragma unroll
+  for (int k = 0; k < kMaxTaps - 1 + kConvTokens; ++k) {
+    const int t = t0 - K + k;
+    rows[k] = (k < K + kConvTokens && t >= 0 && t < n) ? *reinterpret_cast<const f32x4*>(x + (size_t)t * ldx + c) : zero;
+  }
+#pragma unroll
+  for (int i = 0; i < kConvTokens; ++i)
+    cur[i] = t0 + i < n ? *reinterpret_cast<const f32x4*>(x + (size_t)(t0 + i) * ldx + c) : zero;
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) wv[j] = j < taps ? *reinterpret_cast<const f32x4*>(w + (size_t)j * d + c) : zero;
+#pragma unroll
+  for (int i = 0; i < kConvTokens; ++i) {
+    const int t = t0 + i;
+    if (t >= n) break;
+    const int seq = tok_seq[t], off = t - q_start[seq], first_pos = pos0[seq];
+    const float* st = K > 0 ? state + (size_t)state_slots[seq] * K * d + c : nullptr;
+    f32x4 acc = zero;   // the taps in their order, then x: the sums of the kernel that takes a token a thread
+#pragma unroll
+    for (int j = 0; j < kMaxTaps; ++j) {
+      if (j >= taps) break;
+      const int back = K - j;
+      f32x4 v = zero;
+      if (back == 0) {
+        v = cur[i];
+      } else if (off >= back) {
+        v = rows[i + j];
+      } else if (first_pos + off - back >= 0) {
+        v = *reinterpret_cast<const f32x4*>(st + (size_t)(off + j) * d);   // index position - first_pos + K of the slot
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] = fmaf(wv[j][e], v[e], acc[e]);
+    }
+    store4(out + (size_t)t * ldo + c, cur[i] + acc);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ norm_slices
 struct Slice {
   int col, d, ldo;
@@ -207,6 +262,40 @@ __global__ __launch_bounds__(256) void norm_slices_kernel(const T* __restrict__ 
   const float r = 1.0f / sqrtf(ss / (float)s.d + eps);
   T* o = (T*)s.out + (size_t)blockIdx.x * s.ldo;
   for (int c = threadIdx.x; c < s.d; c += blockDim.x) o[c] = from_f<T>(to_f(row[c]) * r * s.gamma[c]);
+}
+
+// A wave a (row, slice), the slice in registers: runs of whole words, at most 4 words a lane.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_slices_words_kernel(const T* __restrict__ in, int ld, int n, Slice s0, Slice s1,
+                                                                float eps) {
+  constexpr int N = Word<T>::N;
+  const Slice s = blockIdx.y == 0 ? s0 : s1;
+  const int r = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (r >= n) return;
+  const T* row = in + (size_t)r * ld + s.col;
+  float v[4][N];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = (lane + i * kWave) * N;
+    if (c < s.d) {
+      load_word(row + c, v[i]);
+#pragma unroll
+      for (int e = 0; e < N; ++e) ss = fmaf(v[i][e], v[i][e], ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float scale = 1.0f / sqrtf(ss / (float)s.d + eps);
+  T* o = (T*)s.out + (size_t)r * s.ldo;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = (lane + i * kWave) * N;
+    if (c < s.d) {
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[i][e] = v[i][e] * scale * s.gamma[c + e];
+      store_word(o + c, v[i]);
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------------ cache write
@@ -690,6 +779,13 @@ extern "C" int gb_time_conv(const float* x, int ldx, const float* w, int taps, f
   const long long count = (long long)n * d;
   GB_REQUIRE(grid_fits(count, 256), "time_conv: too many elements");
   if (d % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && words16(x) && words16(out) && words16(state) && words16(w) && (d + 1023) / 1024 < 65536) {
+    if (taps >= 1 && !single && n >= 256) {
+      const dim3 grid44((unsigned)((n + kConvTokens - 1) / kConvTokens), (unsigned)((d + 1023) / 1024));
+      GB_BY_DTYPE(dtype, "time_conv",
+                  hipLaunchKernelGGL(time_conv4x4_kernel<TT>, grid44, dim3(256), 0, stream, x, ldx, w, taps, state, tok_seq,
+                                     q_start, pos0, state_slots, (TT*)out, ldo, n, d))
+      return launched("time_conv");
+    }
     const dim3 grid4((unsigned)n, (unsigned)((d + 1023) / 1024));
     GB_BY_DTYPE(dtype, "time_conv",
                 hipLaunchKernelGGL(time_conv4_kernel<TT>, grid4, dim3(256), 0, stream, x, ldx, w, taps, state, tok_seq, q_start,
@@ -715,6 +811,16 @@ extern "C" int gb_norm_slices(const void* in, int dtype, int ld, int n, float ep
   GB_REQUIRE(n <= 0x7fffffff, "norm_slices: too many rows");
   if (n == 0) return 0;
   const Slice s0{col0, d0, ldo0, gamma0, out0}, s1{col1, d1, ldo1, gamma1, out1};
+  const int wn = dtype == kBF16 ? 8 : 4;
+  auto in_words = [&](const Slice& s) {
+    return s.d == 0 || (s.col % wn == 0 && s.d % wn == 0 && s.d <= 4 * kWave * wn && s.ldo % wn == 0 && words16(s.out));
+  };
+  if (ld % wn == 0 && words16(in) && in_words(s0) && in_words(s1)) {
+    const dim3 gridw((unsigned)((n + 3) / 4), d1 > 0 ? 2u : 1u);
+    GB_BY_DTYPE(dtype, "norm_slices",
+                hipLaunchKernelGGL(norm_slices_words_kernel<TT>, gridw, dim3(256), 0, stream, (const TT*)in, ld, n, s0, s1, eps))
+    return launched("norm_slices");
+  }
   const dim3 grid((unsigned)n, d1 > 0 ? 2u : 1u);
   GB_BY_DTYPE(dtype, "norm_slices",
               hipLaunchKernelGGL(norm_slices_kernel<TT>, grid, dim3(256), 0, stream, (const TT*)in, ld, s0, s1, eps))

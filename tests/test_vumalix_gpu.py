@@ -77,6 +77,40 @@ def test_the_convolution_of_the_residual_in_portions(d, taps, dtype):
         assert torch.all(state[1] == 55.0) and torch.all(state[4] == 55.0)   # nobody else's slot was touched
 
 
+@pytest.mark.parametrize("d, taps, dtype", [(64, 4, torch.bfloat16), (40, 8, torch.float32), (128, 2, torch.float32), (8, 1, torch.bfloat16)])
+def test_the_convolution_in_long_portions(d, taps, dtype):
+    """Steps of several hundred rows (the kernel that takes four tokens a thread): three requests whose portions begin and
+    end at any token of a group of four, a second step that reads what the first left in the slots, and a request that
+    joins with a portion shorter than the convolution."""
+    from glassbox_amd import ops
+    torch.manual_seed(3 * d + taps)
+    lens = {0: 571, 1: 333, 2: 263}
+    cuts = {0: (301, 270), 1: (2, 331), 2: (0, 263)}
+    slots = {0: 1, 1: 4, 2: 0}
+    w = torch.randn(d, taps).float()
+    state = torch.full((5, max(taps - 1, 1), d), 55.0, device=DEV) if taps > 1 else None
+    data = {r: torch.randn(T, d).float().to(F64) for r, T in lens.items()}
+    want = {r: pv.mixer_input(x, w.to(F64)) for r, x in data.items()}
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    done = {r: 0 for r in lens}
+    for step in range(2):
+        rows = [(r, done[r], done[r] + cuts[r][step]) for r in lens if cuts[r][step]]
+        ctx = _step_ctx(rows, slots)
+        x = _dev(torch.cat([data[r][a:b] for r, a, b in rows], 0))
+        out = torch.full((x.shape[0], d + 4), 9.0, dtype=dtype, device=DEV)[:, :d]
+        ops.time_conv(x, _dev(w.t()), state, ctx, out)
+        got, at = out.cpu().to(F64), 0
+        for r, a, b in rows:
+            assert (got[at:at + b - a] - want[r][a:b]).abs().max() < tol * max(1.0, float(want[r].abs().max())), (step, r)
+            at += b - a
+            done[r] = b
+            if state is not None:
+                kept = state[slots[r]].cpu().to(F64)
+                assert all(torch.equal(kept[i], data[r][b - (taps - 1) + i]) for i in range(taps - 1) if b - (taps - 1) + i >= 0)
+    if state is not None:
+        assert torch.all(state[2] == 55.0) and torch.all(state[3] == 55.0)
+
+
 # ------------------------------------------------------------------------------------------ norms and the polynomial
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norms_of_slices_the_polynomial_the_gate_and_the_normed_add(dtype):
