@@ -93,8 +93,13 @@ class VumalixConfig(ModelConfig):
             j = layer.get("weights_of")
             if j is None:
                 continue
-            if j >= len(checked) or j == i or checked[j].get("weights_of") is not None:
-                raise ConfigError(f"layers[{i}]: weights_of names layer {j}, which must be another layer with tensors of its own")
+            seen = {i}
+            while j is not None and j < len(checked) and j not in seen:   # a layer that itself uses another's: follow it
+                seen.add(j)
+                last, j = j, checked[j].get("weights_of")
+            if j is not None:
+                raise ConfigError(f"layers[{i}]: weights_of must lead to another layer with tensors of its own, and leads to layer {j}")
+            j = last
             if (checked[j]["type"], checked[j]["mixer"], checked[j]["mlp"]) != (layer["type"], layer["mixer"], layer["mlp"]):
                 raise ConfigError(f"layers[{i}] uses the tensors of layer {j} and must equal it in everything else")
         eps = _num("norm", _obj(where, raw, "norm", True), "eps")
@@ -120,5 +125,6 @@ class VumalixConfig(ModelConfig):
 
     def owner(self, i: int) -> int:
         """The layer whose tensors layer i uses."""
-        j = self.layers[i].get("weights_of")
-        return i if j is None else j
+        while self.layers[i].get("weights_of") is not None:
+            i = self.layers[i]["weights_of"]
+        return i

@@ -186,10 +186,13 @@ def test_the_configuration_is_checked_key_by_key():
         else:
             at[path[-1]] = value
         return raw
+    # a layer may name one that itself uses another's tensors: the chain is followed to the layer that owns them
+    assert [config_from_dict(broken(("layers", 3, "weights_of"), 2)).owner(i) for i in range(5)] == [0, 1, 0, 0, 4]
     for path, value, word in ((("layers", 0, "type"), "conv", "type"), (("layers", 1, "mixer", "kv_heads"), 3, "kv_heads"),
                               (("layers", 0, "mixer", "rot", "dims"), 7, "dims"), (("layers", 0, "mixer", "kv_rank"), None, "kv_rank"),
                               (("layers", 1, "mixer", "diff"), None, "diff"), (("layers", 1, "mixer", "q_temp", "every"), 0, "every"),
-                              (("layers", 2, "weights_of"), 3, "weights_of"), (("layers", 2, "weights_of"), 1, "equal"),
+                              (("layers", 3, "weights_of"), 3, "weights_of"), (("layers", 3, "weights_of"), 7, "weights_of"),
+                              (("layers", 2, "weights_of"), 1, "equal"),
                               (("layers", 2, "mixer", "scale"), 0.7, "equal"), (("norm",), None, "norm"),
                               (("layers", 1, "mlp", "kind"), "moe", "kind"), (("canon", "taps"), 0, "taps"), (("layers", 0, "mixer", "rot"), None, "rot")):
         with pytest.raises(ConfigError, match=word):
