@@ -143,12 +143,24 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
   }
 }
 
+// The result rows are bfloat16, or float32 for a caller that goes on in 32-bit with them (a difference of two heads'
+// results, which rounding each first would spoil).
+__device__ __forceinline__ void store_out(bf16* p, float v) { *p = (bf16)v; }
+__device__ __forceinline__ void store_out(float* p, float v) { *p = v; }
+__device__ __forceinline__ void store_out4(bf16* p, const f32x4& v) {
+  bf16x4 o;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) o[r] = (bf16)v[r];
+  *reinterpret_cast<bf16x4*>(p) = o;
+}
+__device__ __forceinline__ void store_out4(float* p, const f32x4& v) { *reinterpret_cast<f32x4*>(p) = v; }
+
 // ----------------------------------------------------------------------------- decode
 // grid (chunks, kv heads, requests); request s is row s of q and out, at position positions[s].
 // WAVES waves take 64 keys each in turn; dynamic LDS holds their partial results for the merge:
 // WAVES * (32 + HD * G) floats, G the query heads per kv head.
-template <int HD, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+template <int HD, int WAVES, typename OT>
+__global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restrict__ q, int q_stride, OT* __restrict__ out,
                                                             int out_stride, float* __restrict__ ws_acc,
                                                             float* __restrict__ ws_ml, const int32_t* __restrict__ positions,
                                                             const int32_t* __restrict__ tables, int table_stride,
@@ -216,7 +228,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
     }
     const int head = kvh * G + cc;
     if (splits == 1) {
-      out[(size_t)s * out_stride + (size_t)head * HD + d] = (bf16)(val / L);
+      store_out(out + (size_t)s * out_stride + (size_t)head * HD + d, val / L);
     } else {
       const size_t slot = ((size_t)s * nh + head) * splits + split;
       ws_acc[slot * HD + d] = val;
@@ -234,8 +246,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
 // asked for at once (a chunk's maximum and sum by thread k, the first partial results of the thread's dimension),
 // and the maximum over the chunks and the sum of their weights are taken wave by wave, not by one thread in turn:
 // the kernel is short, and round trips and serial loops are what it consists of.
+template <typename OT>
 __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
-                                                            bf16* __restrict__ out, int out_stride,
+                                                            OT* __restrict__ out, int out_stride,
                                                             const int32_t* __restrict__ positions, int nh, int hd, int window,
                                                             int keep, int chunk, int splits) {
   constexpr int EARLY = 4;           // partial results a thread asks for before it knows their weights
@@ -291,7 +304,7 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restr
     float total = 0.f;
     for (int g = 0; g < groups; ++g) total += sm_part[g * hd + tid];
     const float l = ((sm_sum[0] + sm_sum[1]) + sm_sum[2]) + sm_sum[3];
-    out[(size_t)s * out_stride + (size_t)head * hd + tid] = (bf16)(total / l);
+    store_out(out + (size_t)s * out_stride + (size_t)head * hd + tid, total / l);
   }
 }
 
@@ -472,8 +485,8 @@ __device__ __forceinline__ BlockRange block_range(int t0, int qlen, int p0, int 
   return r;
 }
 
-template <int HD>
-__device__ __forceinline__ void store_block(const f32x16 (&acc)[(HD + 31) / 32], float l, bf16* __restrict__ orow, int g) {
+template <int HD, typename OT>
+__device__ __forceinline__ void store_block(const f32x16 (&acc)[(HD + 31) / 32], float l, OT* __restrict__ orow, int g) {
   const float inv = 1.0f / l;
 #pragma unroll
   for (int b = 0; b < (HD + 31) / 32; ++b)
@@ -481,10 +494,10 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[(HD + 31) / 32],
     for (int jj = 0; jj < 4; ++jj) {
       const int d0 = 32 * b + 8 * jj + 4 * g;
       if (32 * b + 32 <= HD || d0 < HD) {
-        bf16x4 o;
+        f32x4 o;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = (bf16)(acc[b][4 * jj + r] * inv);
-        *reinterpret_cast<bf16x4*>(orow + d0) = o;
+        for (int r = 0; r < 4; ++r) o[r] = acc[b][4 * jj + r] * inv;
+        store_out4(orow + d0, o);
       }
     }
 }
@@ -513,7 +526,8 @@ __device__ __forceinline__ void store_part(const f32x16 (&acc)[(HD + 31) / 32], 
 }
 
 // Adds the parts in their order: one workgroup of HD threads per (row, head).
-__global__ void prefill_parts_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
+template <typename OT>
+__global__ void prefill_parts_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, OT* __restrict__ out,
                                      int out_stride, int first_row, int n_rows, int nh, int hd, int parts, float c) {
   const int row = blockIdx.x / nh, head = blockIdx.x % nh, d = threadIdx.x;
   if (d >= hd) return;
@@ -527,7 +541,7 @@ __global__ void prefill_parts_kernel(const float* __restrict__ part_acc, const f
     val += part_acc[(k * stride + cell) * hd + d] * f;
     l += part_ml[(k * stride + cell) * 2 + 1] * f;
   }
-  out[(size_t)(first_row + row) * out_stride + (size_t)head * hd + d] = (bf16)(val / l);
+  store_out(out + (size_t)(first_row + row) * out_stride + (size_t)head * hd + d, val / l);
 }
 
 // The waves of a group that shared a block's keys add up their maxima, sums and accumulators into wave 0 through LDS,
@@ -574,8 +588,8 @@ __device__ __forceinline__ void hand_over(float& m, float& l, f32x16 (&acc)[DB],
 // blocks w and n-1-w of 32 tokens.  SPLIT waves share a pair: they take its tiles of 64 keys in turn, and at the
 // end the others hand their sums to the first through LDS.  One wave a pair is best when the pairs alone give
 // every SIMD a wave; short portions and few heads do not, and then the keys are what is left to divide.
-template <int HD, int QB, int PAIRS, int SPLIT>
-__global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+template <int HD, int QB, int PAIRS, int SPLIT, typename OT>
+__global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf16* __restrict__ q, int q_stride, OT* __restrict__ out,
                                                       int out_stride, const int32_t* __restrict__ q_start,
                                                       const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
                                                       int seq_base, const int32_t* __restrict__ tables, int table_stride,
@@ -707,7 +721,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
         store_part<HD>(acc[qb], m[qb], total, part_acc + cell * HD, part_ml + cell * 2, g);
         continue;
       }
-      store_block<HD>(acc[qb], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+      store_block<HD, OT>(acc[qb], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
     }
   } else {
     for (int which = 0; which < (has_second ? 2 : 1); ++which) {
@@ -747,7 +761,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
         const size_t cell = ((size_t)part * n_rows + (row0 + tok - first_row)) * nh + head;
         store_part<HD>(acc[0], m[0], total, part_acc + cell * HD, part_ml + cell * 2, g);
       } else if (valid) {
-        store_block<HD>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+        store_block<HD, OT>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
       }
     }
   }
@@ -762,11 +776,11 @@ extern "C" int gb_attention_supported_head_size(int hd) { return hd >= 16 && hd 
 // q, out: rows 0 .. n_decode-1 are the decoding requests (one row each).  ws_acc must hold
 // n_decode*nh*splits*hd floats and ws_ml n_decode*nh*splits*2, with splits = ceil(max_context / chunk).
 // keep_first > 0 (with a window): keys 0 .. keep_first-1 are read wherever the window has moved past them.
-extern "C" int gb_attention_decode_bf16_keep(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
-                                             const int32_t* positions, const int32_t* tables, int table_stride,
-                                             const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
-                                             int page_size, float scale, int window, int keep_first, int chunk,
-                                             int max_context, hipStream_t stream) {
+template <typename OT>
+static int decode_launch(const void* q, int q_stride, OT* out, int out_stride, void* ws_acc, void* ws_ml,
+                         const int32_t* positions, const int32_t* tables, int table_stride, const void* k_pages,
+                         const void* v_pages, int n_decode, int nh, int nkv, int hd, int page_size, float scale, int window,
+                         int keep_first, int chunk, int max_context, hipStream_t stream) {
   GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_decode: kept first keys go with a window");
   GB_REQUIRE(n_decode >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_decode: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_decode: head size %d is not a multiple of 16 up to 128", hd);
@@ -790,11 +804,11 @@ extern "C" int gb_attention_decode_bf16_keep(const void* q, int q_stride, void* 
 #define GB_CASE(HD)                                                                                                         \
   if (hd == HD) {                                                                                                           \
     if (waves == 16)                                                                                                        \
-      hipLaunchKernelGGL((decode_kernel<HD, 16>), grid, block, lds, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride, \
+      hipLaunchKernelGGL((decode_kernel<HD, 16, OT>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride, \
                          (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
                          (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits);                           \
     else                                                                                                                    \
-      hipLaunchKernelGGL((decode_kernel<HD, 4>), grid, block, lds, stream, (const bf16*)q, q_stride, (bf16*)out, out_stride,  \
+      hipLaunchKernelGGL((decode_kernel<HD, 4, OT>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride,  \
                          (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
                          (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits);                           \
   }
@@ -803,11 +817,31 @@ extern "C" int gb_attention_decode_bf16_keep(const void* q, int q_stride, void* 
   if (int rc = launched("attention_decode")) return rc;
   if (splits > 1) {
     GB_REQUIRE(splits <= 256, "attention_decode: %d chunks are more than the 256 the second pass combines", splits);
-    hipLaunchKernelGGL(decode_reduce_kernel, dim3(n_decode * nh), dim3(256), 0, stream, (const float*)ws_acc,
-                       (const float*)ws_ml, (bf16*)out, out_stride, positions, nh, hd, window, keep_first, chunk, splits);
+    hipLaunchKernelGGL(decode_reduce_kernel<OT>, dim3(n_decode * nh), dim3(256), 0, stream, (const float*)ws_acc,
+                       (const float*)ws_ml, out, out_stride, positions, nh, hd, window, keep_first, chunk, splits);
     return launched("attention_decode_reduce");
   }
   return 0;
+}
+
+extern "C" int gb_attention_decode_bf16_keep(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
+                                             const int32_t* positions, const int32_t* tables, int table_stride,
+                                             const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
+                                             int page_size, float scale, int window, int keep_first, int chunk,
+                                             int max_context, hipStream_t stream) {
+  return decode_launch<bf16>(q, q_stride, (bf16*)out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k_pages, v_pages,
+                             n_decode, nh, nkv, hd, page_size, scale, window, keep_first, chunk, max_context, stream);
+}
+
+// The same with float32 result rows (out_stride in floats, rows 16-byte aligned): q, keys and values stay bfloat16.
+extern "C" int gb_attention_decode_bf16_out32(const void* q, int q_stride, void* out, int out_stride, void* ws_acc,
+                                              void* ws_ml, const int32_t* positions, const int32_t* tables, int table_stride,
+                                              const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
+                                              int page_size, float scale, int window, int keep_first, int chunk,
+                                              int max_context, hipStream_t stream) {
+  GB_REQUIRE((uintptr_t)out % 16 == 0, "attention_decode: float32 result rows must be 16-byte aligned");
+  return decode_launch<float>(q, q_stride, (float*)out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k_pages,
+                              v_pages, n_decode, nh, nkv, hd, page_size, scale, window, keep_first, chunk, max_context, stream);
 }
 
 extern "C" int gb_attention_decode_bf16(const void* q, int q_stride, void* out, int out_stride, void* ws_acc, void* ws_ml,
@@ -914,12 +948,12 @@ extern "C" int gb_attention_prefill_parts(int max_q_len, int max_context, int nh
 // q and out that the portions occupy (contiguous); part_ws: float32 workspace of part_floats elements, needed if
 // gb_attention_prefill_parts says so.
 // keep_first > 0 (with a window): keys 0 .. keep_first-1 are read wherever the window has moved past them.
-extern "C" int gb_attention_prefill_bf16_keep(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
-                                              const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs,
-                                              int max_q_len, int max_context, const int32_t* tables, int table_stride,
-                                              const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
-                                              float scale, int window, int keep_first, int first_row, int n_rows,
-                                              float* part_ws, long long part_floats, hipStream_t stream) {
+template <typename OT>
+static int prefill_launch(const void* q, int q_stride, OT* out, int out_stride, const int32_t* q_start, const int32_t* q_len,
+                          const int32_t* pos0, int seq_base, int n_seqs, int max_q_len, int max_context, const int32_t* tables,
+                          int table_stride, const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
+                          float scale, int window, int keep_first, int first_row, int n_rows, float* part_ws,
+                          long long part_floats, hipStream_t stream) {
   GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_prefill: kept first keys go with a window");
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_prefill: head size %d is not a multiple of 16 up to 128", hd);
@@ -943,7 +977,7 @@ extern "C" int gb_attention_prefill_bf16_keep(const void* q, int q_stride, void*
   }
   const dim3 grid((max_q_len + 64 * per_group - 1) / (64 * per_group) * parts, nh, n_seqs), block(64 * per_group * split);
 #define GB_LAUNCH(HD, QB, PAIRS, SPLIT)                                                                                     \
-  hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT>), grid, block, 0, stream, (const bf16*)q, q_stride, (bf16*)out, \
+  hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT, OT>), grid, block, 0, stream, (const bf16*)q, q_stride, out, \
                      out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages,               \
                      (const bf16*)v_pages, nh, nkv, page_shift, scale, window, keep_first, part_acc, part_ml, parts, first_row, \
                      n_rows)
@@ -965,11 +999,35 @@ extern "C" int gb_attention_prefill_bf16_keep(const void* q, int q_stride, void*
 #undef GB_LAUNCH
   if (int rc = launched("attention_prefill")) return rc;
   if (parts > 1) {
-    hipLaunchKernelGGL(prefill_parts_kernel, dim3((unsigned)(n_rows * nh)), dim3((hd + 63) / 64 * 64), 0, stream, part_acc, part_ml,
-                       (bf16*)out, out_stride, first_row, n_rows, nh, hd, parts, scale * 1.4426950408889634f);
+    hipLaunchKernelGGL(prefill_parts_kernel<OT>, dim3((unsigned)(n_rows * nh)), dim3((hd + 63) / 64 * 64), 0, stream, part_acc,
+                       part_ml, out, out_stride, first_row, n_rows, nh, hd, parts, scale * 1.4426950408889634f);
     return launched("attention_prefill (second pass)");
   }
   return 0;
+}
+
+extern "C" int gb_attention_prefill_bf16_keep(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
+                                              const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs,
+                                              int max_q_len, int max_context, const int32_t* tables, int table_stride,
+                                              const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
+                                              float scale, int window, int keep_first, int first_row, int n_rows,
+                                              float* part_ws, long long part_floats, hipStream_t stream) {
+  return prefill_launch<bf16>(q, q_stride, (bf16*)out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, max_context,
+                              tables, table_stride, k_pages, v_pages, nh, nkv, hd, page_size, scale, window, keep_first, first_row,
+                              n_rows, part_ws, part_floats, stream);
+}
+
+// The same with float32 result rows (out_stride in floats, rows 16-byte aligned).
+extern "C" int gb_attention_prefill_bf16_out32(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
+                                               const int32_t* q_len, const int32_t* pos0, int seq_base, int n_seqs,
+                                               int max_q_len, int max_context, const int32_t* tables, int table_stride,
+                                               const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
+                                               float scale, int window, int keep_first, int first_row, int n_rows,
+                                               float* part_ws, long long part_floats, hipStream_t stream) {
+  GB_REQUIRE((uintptr_t)out % 16 == 0, "attention_prefill: float32 result rows must be 16-byte aligned");
+  return prefill_launch<float>(q, q_stride, (float*)out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len,
+                               max_context, tables, table_stride, k_pages, v_pages, nh, nkv, hd, page_size, scale, window,
+                               keep_first, first_row, n_rows, part_ws, part_floats, stream);
 }
 
 extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out, int out_stride, const int32_t* q_start,
@@ -986,5 +1044,7 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
 GB_TAPED(gb_attention_decode_bf16_keep)
 GB_TAPED(gb_attention_prefill_bf16_keep)
+GB_TAPED(gb_attention_decode_bf16_out32)
+GB_TAPED(gb_attention_prefill_bf16_out32)
 GB_TAPED(gb_attention_decode_bf16)
 GB_TAPED(gb_attention_prefill_bf16)

@@ -541,8 +541,8 @@ __global__ __launch_bounds__(4 * kWave) void diff_heads_words_kernel(
 
 // ------------------------------------------------------------------------------------------------ diff_combine
 // Sixteen lanes a (token, head): att holds 2 H heads of hd columns, the maps of head h in heads 2 h and 2 h + 1.
-template <typename T>
-__global__ __launch_bounds__(4 * kWave) void diff_combine_kernel(const T* __restrict__ att, int lda, int hd,
+template <typename AT, typename T>
+__global__ __launch_bounds__(4 * kWave) void diff_combine_kernel(const AT* __restrict__ att, int lda, int hd,
                                                                  const float* __restrict__ lambda, float mult, float eps,
                                                                  T* __restrict__ out, int ldo, long long units, int H,
                                                                  int vdim) {
@@ -550,8 +550,8 @@ __global__ __launch_bounds__(4 * kWave) void diff_combine_kernel(const T* __rest
   const long long unit = ((long long)blockIdx.x * blockDim.x + threadIdx.x) / kLanes;
   const bool live = unit < units;
   const int t = live ? (int)(unit / H) : 0, h = live ? (int)(unit % H) : 0;
-  const T* a1 = att + (size_t)t * lda + (size_t)(2 * h) * hd;
-  const T* a2 = a1 + hd;
+  const AT* a1 = att + (size_t)t * lda + (size_t)(2 * h) * hd;
+  const AT* a2 = a1 + hd;
   const float lam = lambda[0];
   float ss = 0.f;
   if (live)
@@ -904,17 +904,24 @@ extern "C" int gb_diff_heads(const void* proj, int dtype, int ld, const float* w
   return launched("diff_heads");
 }
 
-// att [n, lda]: 2 H heads of hd columns; lambda: one float32 on the device; out [n, ldo]: H heads of vdim.
-extern "C" int gb_diff_combine(const void* att, int dtype, int lda, int hd, const float* lambda, float mult, float eps,
-                               void* out, int ldo, int n, int H, int vdim, hipStream_t stream) {
+// att [n, lda]: 2 H heads of hd columns, of the result's type or float32; lambda: one float32 on the device;
+// out [n, ldo]: H heads of vdim.
+extern "C" int gb_diff_combine(const void* att, int att_dtype, int lda, int hd, const float* lambda, float mult, float eps,
+                               void* out, int dtype, int ldo, int n, int H, int vdim, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && H > 0 && vdim > 0 && hd >= vdim && lda >= 2 * H * hd && ldo >= H * vdim && lambda,
              "diff_combine: bad sizes heads=%d vdim=%d head columns=%d", H, vdim, hd);
+  GB_REQUIRE(att_dtype == dtype || att_dtype == kF32, "diff_combine: the heads are of the result's type or float32");
   if (n == 0) return 0;
   const long long units = (long long)n * H;
   GB_REQUIRE(grid_fits(units * kLanes, 256), "diff_combine: too many heads");
   const dim3 grid((unsigned)((units * kLanes + 255) / 256));
+  if (att_dtype == kF32 && dtype == kBF16) {
+    hipLaunchKernelGGL((diff_combine_kernel<float, bf16>), grid, dim3(256), 0, stream, (const float*)att, lda, hd, lambda, mult,
+                       eps, (bf16*)out, ldo, units, H, vdim);
+    return launched("diff_combine");
+  }
   GB_BY_DTYPE(dtype, "diff_combine",
-              hipLaunchKernelGGL(diff_combine_kernel<TT>, grid, dim3(256), 0, stream, (const TT*)att, lda, hd, lambda, mult,
+              hipLaunchKernelGGL((diff_combine_kernel<TT, TT>), grid, dim3(256), 0, stream, (const TT*)att, lda, hd, lambda, mult,
                                  eps, (TT*)out, ldo, units, H, vdim))
   return launched("diff_combine");
 }

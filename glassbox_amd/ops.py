@@ -80,8 +80,8 @@ _SIGS = {
         "gb_latent_heads": [_vp, _i, _vp, _i, _vp, _i, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
         # proj, dtype, ld, wq, wk, eps, coef, every, positions, out, ldo, hd, slots, k, v, page, n, H, G, dim, vdim, stream
         "gb_diff_heads": [_vp, _i, _i, _vp, _vp, _f, _f, _i, _vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-        # att, dtype, lda, hd, lambda, mult, eps, out, ldo, n, H, vdim, stream
-        "gb_diff_combine": [_vp, _i, _i, _i, _vp, _f, _f, _vp, _i, _i, _i, _i, _vp],
+        # att, its dtype, lda, hd, lambda, mult, eps, out, its dtype, ldo, n, H, vdim, stream
+        "gb_diff_combine": [_vp, _i, _i, _i, _vp, _f, _f, _vp, _i, _i, _i, _i, _i, _vp],
         # att, lda, hd, gate, ldg, dtype, out, ldo, n, H, vdim, stream
         "gb_gate_heads": [_vp, _i, _i, _vp, _i, _i, _vp, _i, _i, _i, _i, _vp],
         # z, ldz, coef, eps, out, ldo, dtype, n, d, stream
@@ -169,6 +169,11 @@ _SIGS = {
                                           _i, _i, _vp],
         "gb_attention_prefill_bf16_keep": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                                            _f, _i, _i, _i, _i, _vp, C.c_longlong, _vp],
+        # the same two with float32 result rows
+        "gb_attention_decode_bf16_out32": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
+                                           _i, _i, _vp],
+        "gb_attention_prefill_bf16_out32": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
+                                            _f, _i, _i, _i, _i, _vp, C.c_longlong, _vp],
     },
     "sampling": {
         "gb_argmax": [_vp, _vp, _i, _i, _vp],
@@ -1010,15 +1015,18 @@ def diff_heads(proj: torch.Tensor, w_q: torch.Tensor, w_k: torch.Tensor, eps: fl
 def diff_combine(att: torch.Tensor, head_cols: int, lam: torch.Tensor, mult: float, eps: float, out: torch.Tensor,
                  n_heads: int, vdim: int) -> None:
     """out[:, h] = mult * o / sqrt(mean(o^2) + eps), o = a1 - lam * a2, where a1, a2 are heads 2 h and 2 h + 1 of ``att``
-    ([n, 2 heads * head_cols]) cut to vdim columns and ``lam`` is one float32 on the device; ``out`` [n, heads * vdim]."""
+    ([n, 2 heads * head_cols], of out's type or float32) cut to vdim columns and ``lam`` is one float32 on the device;
+    ``out`` [n, heads * vdim]."""
     _dev(att, lam, out)
-    n, dt = att.shape[0], att.dtype
-    lda = _act_rows(att, dt, 2 * n_heads * head_cols, "att")
+    n, dt = att.shape[0], out.dtype
+    if att.dtype not in (dt, torch.float32):
+        raise KernelError("diff_combine: att must have out's type or be float32")
+    lda = _act_rows(att, att.dtype, 2 * n_heads * head_cols, "att")
     ldo = _act_rows(out, dt, n_heads * vdim, "out")
     _f32_rows(lam, (1,), "lam")
     lib = _lib("headmix")
     _launch(lib, lib.gb_diff_combine, _p(att), dtype_code(att), lda, int(head_cols), _p(lam), float(mult), float(eps),
-            _p(out), ldo, n, n_heads, vdim, _stream())
+            _p(out), dtype_code(out), ldo, n, n_heads, vdim, _stream())
 
 
 def gate_heads(att: torch.Tensor, head_cols: int, gate: torch.Tensor, out: torch.Tensor, n_heads: int, vdim: int) -> None:
@@ -1579,8 +1587,8 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
     k_pages, v_pages = cache.k_pages, cache.v_pages
     _dev(q, out, k_pages, v_pages)
     _, nkv, page, hd = _check_pages(k_pages, v_pages, torch.bfloat16, "attention_decode")
-    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or q.shape[1] != n_heads * hd:
-        raise KernelError("attention_decode: q and out must be bfloat16 [n, heads * head size]")
+    if q.dtype != torch.bfloat16 or out.dtype not in (torch.bfloat16, torch.float32) or q.shape[1] != n_heads * hd:
+        raise KernelError("attention_decode: q must be bfloat16 [n, heads * head size], out bfloat16 or float32")
     tables = ctx.tables[cache.group]
     max_context = int(ctx.host["max_context"])
     chunk = decode_chunk(n_dec, nkv, max_context)
@@ -1588,8 +1596,8 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
     ws_acc = ctx.buffer("attn_ws_acc", (n_dec * n_heads * splits * hd,), torch.float32)
     ws_ml = ctx.buffer("attn_ws_ml", (n_dec * n_heads * splits * 2,), torch.float32)
     lib = _lib("attention_bf16")
-    if keep_first:
-        _launch(lib, lib.gb_attention_decode_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
+    if keep_first or out.dtype == torch.float32:
+        _launch(lib, lib.gb_attention_decode_bf16_out32 if out.dtype == torch.float32 else lib.gb_attention_decode_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
                 _p(ctx.positions), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_dec, n_heads, nkv, hd, page,
                 float(scale), int(window), int(keep_first), chunk, max_context, _stream())
         return
@@ -1611,8 +1619,8 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     k_pages, v_pages = cache.k_pages, cache.v_pages
     _dev(q, out, k_pages, v_pages)
     _, nkv, page, hd = _check_pages(k_pages, v_pages, torch.bfloat16, "attention_prefill")
-    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or q.shape[1] != n_heads * hd:
-        raise KernelError("attention_prefill: q and out must be bfloat16 [n, heads * head size]")
+    if q.dtype != torch.bfloat16 or out.dtype not in (torch.bfloat16, torch.float32) or q.shape[1] != n_heads * hd:
+        raise KernelError("attention_prefill: q must be bfloat16 [n, heads * head size], out bfloat16 or float32")
     tables = ctx.tables[cache.group]
     lib = _lib("attention_bf16")
     max_q, max_ctx = int(ctx.host["max_q_len"]), int(ctx.host["max_context"])
@@ -1621,8 +1629,8 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     first_row, n_rows = n_dec, q.shape[0] - n_dec
     parts = _prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
     ws = ctx.buffer("attn_parts", (parts * n_rows * n_heads * (hd + 2),), torch.float32) if parts > 1 else None
-    if keep_first:
-        _launch(lib, lib.gb_attention_prefill_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
+    if keep_first or out.dtype == torch.float32:
+        _launch(lib, lib.gb_attention_prefill_bf16_out32 if out.dtype == torch.float32 else lib.gb_attention_prefill_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
                 _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables), tables.stride(0), _p(k_pages),
                 _p(v_pages), n_heads, nkv, hd, page, float(scale), int(window), int(keep_first), first_row, n_rows, _p(ws),
                 ws.numel() if ws is not None else 0, _stream())

@@ -507,7 +507,10 @@ class DifferentialAttention(Mixer):
         if slots is not None and not direct:
             ops.rope_store(heads, None, None, slots, cache.k_pages, cache.v_pages, 2 * H, G, hc, rotate=False,
                            portions=ctx.portions())
-        att = ctx.buffer("att", (n, 2 * H * hc), ctx.dtype)
+        # the two maps' results stay 32-bit until their difference is taken (where they are close, rounding each
+        # first would be most of what is left), wherever the attention kernels write such rows
+        wide = ctx.dtype == torch.bfloat16 and ctx.tuned and ops.tuned_attention_supports(cache.k_pages, 2 * H, 0, 0)
+        att = ctx.buffer("att32", (n, 2 * H * hc), torch.float32) if wide else ctx.buffer("att", (n, 2 * H * hc), ctx.dtype)
         paged_attention(ctx, heads[:, :2 * H * hc], att, cache, 2 * H, self.scale, 0)
         o = ctx.buffer("diff_o", (n, H * V), ctx.dtype)
         ops.diff_combine(att, hc, self.lam, 1.0 - self.diff, self.eps, o, H, V)
