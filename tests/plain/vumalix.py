@@ -178,8 +178,9 @@ def dense_ff(w, pre: str, eps: float, x: torch.Tensor, rnd=exact) -> torch.Tenso
 # ---------------------------------------------------------------------------------------------- the model
 def layer_owner(cfg: dict, i: int) -> int:
     """The layer whose tensors layer i uses."""
-    j = cfg["layers"][i].get("weights_of")
-    return i if j is None else j
+    while cfg["layers"][i].get("weights_of") is not None:
+        i = cfg["layers"][i]["weights_of"]
+    return i
 
 
 def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], coarse: bool = False,

@@ -5,7 +5,8 @@ another layer's tensors (one layer three times, two layers in turn, none), laten
 a page, across pages and absent, a rotated part of 2 to 32 columns of which all or only some turn, latents narrower and
 wider than the heads, heads whose keys are larger or smaller than their values, heads beyond the matrix-core attention;
 differential attention with one to four query heads a key head, a temperature that steps every 3, 7 or 40 positions or
-is absent, values smaller and larger than two maps; layers without a feed-forward; sizes that are no multiple of 8.
+is absent, values smaller and larger than two maps; layers without a feed-forward, last and in the middle; a chain of
+layers that use another's tensors; sizes that are no multiple of 8.
 Score scales are large enough that single keys carry visible weight.
 """
 from __future__ import annotations
@@ -72,6 +73,23 @@ CASES: Dict[str, dict] = {
         {"type": "latent_attention", "mixer": {"heads": 8, "dim": 48, "rot_dim": 16, "vdim": 64, "q_rank": 96, "kv_rank": 128,
                                                "scale": 0.25, "rot": {"dims": 16, "base": 10000.0}, "mask": {"size": 33}},
          "mlp": {"kind": "dense", "ff": 64}},
+    ]),
+    # three taps; layers without a feed-forward in the middle (the mixer's norm is the layer's last pass); a layer that names
+    # one which itself uses another's tensors; as many key heads as query heads; no temperature; a window of one page
+    "E": dict(architecture="Vumalix", vocab=97, width=72, norm={"eps": 1e-6}, canon={"taps": 3}, layers=[
+        {"type": "latent_attention", "mixer": {"heads": 3, "dim": 16, "rot_dim": 16, "vdim": 24, "q_rank": 40, "kv_rank": 24,
+                                               "scale": 0.3, "rot": {"dims": 16, "base": 500.0}, "mask": {"size": 16}},
+         "mlp": None},
+        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 24, "vdim": 40, "scale": 0.4, "diff": 0.7},
+         "mlp": {"kind": "dense", "ff": 88}},
+        {"type": "latent_attention", "mixer": {"heads": 3, "dim": 16, "rot_dim": 16, "vdim": 24, "q_rank": 40, "kv_rank": 24,
+                                               "scale": 0.3, "rot": {"dims": 16, "base": 500.0}, "mask": {"size": 16}},
+         "mlp": None, "weights_of": 0},
+        {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 24, "vdim": 40, "scale": 0.4, "diff": 0.7},
+         "mlp": {"kind": "dense", "ff": 88}, "weights_of": 1},
+        {"type": "latent_attention", "mixer": {"heads": 3, "dim": 16, "rot_dim": 16, "vdim": 24, "q_rank": 40, "kv_rank": 24,
+                                               "scale": 0.3, "rot": {"dims": 16, "base": 500.0}, "mask": {"size": 16}},
+         "mlp": None, "weights_of": 2},
     ]),
 }
 
