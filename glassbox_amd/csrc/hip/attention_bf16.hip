@@ -21,6 +21,8 @@
 // in a fixed order (waves in LDS, chunks by a second kernel), so the result is the same on every
 // run.  crates/glassbox-core/src/model.rs:285-312 is the formula.
 #include "attention_bf16.h"
+#include <type_traits>
+
 #include "common.h"
 
 #include <mutex>
@@ -63,7 +65,9 @@ __device__ __forceinline__ void reset(Running<HD>& st) {
 // [lo, hi] count for this lane's column; [clamp_lo, clamp_hi] (the same for the whole wave) is a
 // range of keys known to have pages: tiles outside it are redirected to a tile inside it, and all
 // their keys are masked anyway.
-template <int HD>
+// WIDE: the softmax weights enter the value product in two bfloat16 parts, p = hi + lo (two products), which keeps 16
+// bits of them instead of 8: for results that go on in 32-bit.
+template <int HD, bool WIDE = false>
 __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, const bf16* __restrict__ kp,
                                          const bf16* __restrict__ vp, const int32_t* __restrict__ table, int nkv, int kvh,
                                          int P, int kbase, int lo, int hi, int clamp_lo, int clamp_hi, float scale,
@@ -124,11 +128,15 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
     for (int r = 0; r < 4; ++r) st.acc[b][r] *= alpha;
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    bf16x8 pf;
+    bf16x8 pf, pl;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       pf[r] = (bf16)s[2 * u][r];
       pf[4 + r] = (bf16)s[2 * u + 1][r];
+      if (WIDE) {
+        pl[r] = (bf16)(s[2 * u][r] - (float)pf[r]);
+        pl[4 + r] = (bf16)(s[2 * u + 1][r] - (float)pf[4 + r]);
+      }
     }
 #pragma unroll
     for (int b = 0; b < DB; ++b) {
@@ -139,6 +147,7 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
         af[4 + r] = vf[b][2 * u + 1][r];
       }
       st.acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, pf, st.acc[b], 0, 0, 0);
+      if (WIDE) st.acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, pl, st.acc[b], 0, 0, 0);
     }
   }
 }
@@ -168,6 +177,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
                                                             int nkv, int P, float scale, int window, int keep, int chunk,
                                                             int splits) {
   constexpr int KS = (HD + 31) / 32, DB = HD / 16;
+  constexpr bool WIDE = std::is_same<OT, float>::value;
   extern __shared__ float decode_lds[];
   const int s = blockIdx.z, kvh = blockIdx.y, split = blockIdx.x;
   const int G = nh / nkv;
@@ -195,9 +205,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   const int end = min(c0 + chunk, pos + 1);
   for (int kb = c0 + wave * 64; kb < end; kb += 64 * WAVES) {
     // the kept first keys of these 64, then those inside the window (a tile can hold both kinds)
-    if (kb < kept) attend64<HD>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane);
+    if (kb < kept) attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane);
     if (kb + 64 <= lo) continue;
-    attend64<HD>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane);
+    attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane);
   }
   st.l += __shfl_xor(st.l, 16, kWave);
   st.l += __shfl_xor(st.l, 32, kWave);
@@ -387,7 +397,7 @@ __device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][2 * T],
 // registers at a time; as soon as the last block's score products have read kf it is loaded again
 // for the keys from `next`, and vf likewise after the last value products, so that those loads are
 // in flight during the arithmetic in between.
-template <int HD, int QB, int ACT, int T = 2>
+template <int HD, int QB, int ACT, int T = 2, bool WIDE = false>
 __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32x16 (&acc)[QB][(HD + 31) / 32],
                                              const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[T][HD / 16],
                                              bf16x8 (&vf)[(HD + 31) / 32][2 * T], const PageSource& src, int kbase, int next,
@@ -454,11 +464,17 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
     }
 #pragma unroll
     for (int u = 0; u < 2 * T; ++u) {
-      bf16x8 pf;
+      bf16x8 pf, pl;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pf[e] = (bf16)s[u >> 1][8 * (u & 1) + e];
+      for (int e = 0; e < 8; ++e) {
+        pf[e] = (bf16)s[u >> 1][8 * (u & 1) + e];
+        if (WIDE) pl[e] = (bf16)(s[u >> 1][8 * (u & 1) + e] - (float)pf[e]);   // (see attend64)
+      }
 #pragma unroll
-      for (int b = 0; b < DB; ++b) acc[qb][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[b][u], pf, acc[qb][b], 0, 0, 0);
+      for (int b = 0; b < DB; ++b) {
+        acc[qb][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[b][u], pf, acc[qb][b], 0, 0, 0);
+        if (WIDE) acc[qb][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[b][u], pl, acc[qb][b], 0, 0, 0);
+      }
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -599,6 +615,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
                                                       int first_row, int n_rows) {
   // parts > 1: `parts` workgroups share a group's pairs, taking the tiles of keys in turn like the waves of a pair
   // do; each writes its sums to part_acc / part_ml (rows counted from first_row), and prefill_parts_kernel adds them.
+  constexpr bool WIDE = std::is_same<OT, float>::value;   // results that go on in 32-bit: weights in two parts
   constexpr int KS = HD / 16, DB = (HD + 31) / 32;
   // Workgroups go to the chip's eight dies in turn, each die with an L2 of its own.  The ones that
   // land on one die are given consecutive units of work, so that a head's keys and values, which all
@@ -690,18 +707,18 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       while (kb <= range[0].last) {
         const int next = my_next(kb);
         const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));
-        attend64_q32<HD, 2, 3>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep);
+        attend64_q32<HD, 2, 3, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep);
         kb = next;
       }
       while (kb <= range[1].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 2>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep);
+        attend64_q32<HD, 2, 2, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep);
         kb = next;
       }
     } else {
       while (kb <= range[0].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 1>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep);
+        attend64_q32<HD, 2, 1, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep);
         kb = next;
       }
     }
@@ -750,7 +767,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       load_keys<HD, T>(kf, src, key_of(i0), lane);
       load_values<HD, T>(vf, src, key_of(i0), lane);
       for (int i = i0; key_of(i) <= range.last; i += stride)
-        attend64_q32<HD, 1, 1, T>(m, l, acc, q_lds, q_at, kf, vf, src, key_of(i), key_of(i + stride), lo, hi,
+        attend64_q32<HD, 1, 1, T, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, key_of(i), key_of(i + stride), lo, hi,
                                   !range.unmasked(key_of(i), SPAN), c, lane, keep);
       if constexpr (SPLIT > 1) {
         hand_over<DB, SPLIT>(m[0], l[0], acc[0], handed[wave], handed_ml[wave], half, lane, c, which > 0);

@@ -844,6 +844,36 @@ def test_tuned_attention_against_the_plain_kernel(nh, nkv, hd, window, page):
     assert ((out.float() - twin.float()).abs() <= 2 ** -7 * (1 + twin.float().abs())).all()
 
 
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (8, 8, 64, 0), (6, 3, 96, 0), (8, 2, 128, 70), (4, 4, 64, 300), (32, 16, 32, 0)])
+def test_tuned_attention_with_32_bit_result_rows(nh, nkv, hd, window):
+    """The same kernels writing float32 rows (for a caller that goes on in 32-bit, like the difference of two heads):
+    the softmax weights then enter the value product in two bfloat16 parts, so the rows are the float64 formula's on
+    the bfloat16 operands to a few units of the 16th bit, not of the 8th; single tokens, short and long portions, chunks
+    that split."""
+    from types import SimpleNamespace
+    from glassbox_amd import ops
+    q_lens = [1, 1, 1, 1, 1, 5, 70, 16, 1101]
+    ctx_lens = [1, 17, 256, 700, 1025, 5, 300, 16, 1303]
+    k_pages, v_pages, tables, ks, vs = paged_setup(ctx_lens, nkv, hd, 16, seed=hd + nh, dtype=torch.bfloat16)
+    ctx = BareContext(q_lens, ctx_lens, tables, max_context=1400)
+    n = sum(q_lens)
+    q = (rnd(n, nh * hd, seed=11) * 0.7).bfloat16()
+    scale = 1 / math.sqrt(hd)
+    cache = SimpleNamespace(k_pages=to_dev(ops.pack_keys(k_pages)), v_pages=to_dev(v_pages), group=0)
+    out = torch.full((n, nh * hd + 4), 7.0, device=DEV, dtype=torch.float32)[:, :nh * hd]   # rows wider than the heads
+    qd = to_dev(q)
+    ops.attention_decode(qd, out, ctx, cache, nh, scale, window)
+    ops.attention_prefill(qd, out, ctx, cache, nh, scale, window)
+    want = plain_attention_rows(q, ks, vs, ctx.tok_seq, ctx.pos_list, nh, scale, window)
+    err = (out.cpu().double() - want).abs().max(dim=1).values
+    bad = torch.nonzero(err > 2e-4 * (1 + want.abs().max())).flatten().tolist()
+    assert not bad, f"rows {bad[:8]} (request, position) {[(ctx.tok_seq[i], ctx.pos_list[i]) for i in bad[:8]]}: {err[bad[:8]]}"
+    narrow = torch.zeros(n, nh * hd, device=DEV, dtype=torch.bfloat16)
+    ops.attention_decode(qd, narrow, ctx, cache, nh, scale, window)
+    ops.attention_prefill(qd, narrow, ctx, cache, nh, scale, window)
+    assert ((out - narrow.float()).abs() <= 2 ** -6 * (1 + out.abs())).all()
+
+
 @pytest.mark.parametrize("nh,nkv,hd,window", [(32, 32, 64, 0), (32, 8, 48, 0), (32, 4, 16, 100), (32, 32, 64, 200),
                                               (32, 16, 32, 0), (32, 8, 128, 0), (8, 8, 96, 0), (40, 8, 64, 0), (16, 4, 64, 0),
                                               (16, 16, 64, 150)])
