@@ -51,6 +51,7 @@ LIBRARIES: Dict[str, tuple] = {
     "shortconv": ("hip", ["hip/shortconv.hip"], ["hip/common.h"]),
     "moe": ("hip", ["hip/moe.hip"], ["hip/common.h"]),
     "headmix": ("hip", ["hip/headmix.hip"], ["hip/common.h"]),
+    "tanhmix": ("hip", ["hip/tanhmix.hip"], ["hip/common.h"]),
 }
 
 _lock = threading.Lock()

@@ -45,6 +45,22 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// What a mixer may ask of the softmax beyond a window: `span` > 0: positions are cut into runs of `span` from 0 on and a
+// token sees the keys of its own run up to itself (no window then); `softcap` > 0: score = softcap * tanh(score /
+// softcap); `sinks` [nh]: exp(sinks[h]) joins the denominator of head h and has no value.
+struct Extra {
+  int span;
+  float softcap;
+  const float* __restrict__ sinks;
+};
+
+__device__ __forceinline__ int first_key(int pos, int window, int span) {
+  return span > 0 ? pos - pos % span : window > 0 ? max(0, pos - window + 1) : 0;
+}
+
+// tanh by one exponential: 1 - 2 / (1 + e^(2x)); +-1 where the exponential leaves the range
+__device__ __forceinline__ float tanh_fast(float x) { return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * x)); }
+
 template <int HD>
 struct Running {
   float m, l;  // running maximum; this lane's share of the running sum
@@ -71,7 +87,7 @@ template <int HD, bool WIDE = false>
 __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, const bf16* __restrict__ kp,
                                          const bf16* __restrict__ vp, const int32_t* __restrict__ table, int nkv, int kvh,
                                          int P, int kbase, int lo, int hi, int clamp_lo, int clamp_hi, float scale,
-                                         int lane) {
+                                         int lane, float softcap = 0.f) {
   constexpr int KS = (HD + 31) / 32, DB = HD / 16;
   const int j = lane & 15, c = lane >> 4;
   bf16x8 kf[4][KS];
@@ -104,7 +120,9 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int key = kbase + 16 * t + 4 * c + r;
-      s[t][r] = (key >= lo && key <= hi) ? a[r] * scale : -INFINITY;
+      float sc = a[r] * scale;
+      if (softcap > 0.f) sc = softcap * tanh_fast(sc / softcap);   // (the same for the whole wave)
+      s[t][r] = (key >= lo && key <= hi) ? sc : -INFINITY;
       mx = fmaxf(mx, s[t][r]);
     }
   }
@@ -175,7 +193,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
                                                             const int32_t* __restrict__ tables, int table_stride,
                                                             const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh,
                                                             int nkv, int P, float scale, int window, int keep, int chunk,
-                                                            int splits) {
+                                                            int splits, Extra ex) {
   constexpr int KS = (HD + 31) / 32, DB = HD / 16;
   constexpr bool WIDE = std::is_same<OT, float>::value;
   extern __shared__ float decode_lds[];
@@ -185,7 +203,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   float* sm_l = sm_m + WAVES * 16;        // [WAVES][16]
   float* sm_acc = sm_l + WAVES * 16;      // [WAVES][HD][G]
   const int pos = positions[s];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_key(pos, window, ex.span);
   const int c0 = split * chunk;
   const int kept = min(keep, lo);            // keys 0 .. kept-1 are read although the window has passed them
   if (c0 > pos || (c0 + chunk <= lo && c0 >= kept)) return;  // this chunk holds no key of the request
@@ -205,9 +223,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   const int end = min(c0 + chunk, pos + 1);
   for (int kb = c0 + wave * 64; kb < end; kb += 64 * WAVES) {
     // the kept first keys of these 64, then those inside the window (a tile can hold both kinds)
-    if (kb < kept) attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane);
+    if (kb < kept) attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane, ex.softcap);
     if (kb + 64 <= lo) continue;
-    attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane);
+    attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane, ex.softcap);
   }
   st.l += __shfl_xor(st.l, 16, kWave);
   st.l += __shfl_xor(st.l, 32, kWave);
@@ -238,6 +256,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
     }
     const int head = kvh * G + cc;
     if (splits == 1) {
+      if (ex.sinks) L += __expf(ex.sinks[head] - M);
       store_out(out + (size_t)s * out_stride + (size_t)head * HD + d, val / L);
     } else {
       const size_t slot = ((size_t)s * nh + head) * splits + split;
@@ -260,14 +279,14 @@ template <typename OT>
 __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
                                                             OT* __restrict__ out, int out_stride,
                                                             const int32_t* __restrict__ positions, int nh, int hd, int window,
-                                                            int keep, int chunk, int splits) {
+                                                            int keep, int chunk, int splits, Extra ex) {
   constexpr int EARLY = 4;           // partial results a thread asks for before it knows their weights
   __shared__ float sm_f[256];        // chunk k's weight exp(m_k - M)
   __shared__ float sm_part[256];     // [group][dimension]
   __shared__ float sm_top[4], sm_sum[4];
   const int s = blockIdx.x / nh, head = blockIdx.x % nh, tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int pos = positions[s];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_key(pos, window, ex.span);
   // the chunks that hold keys: those of the kept first keys that lie before the window's first chunk, then the window's
   const int first = lo / chunk, last = pos / chunk;
   const int early_chunks = min((min(keep, lo) + chunk - 1) / chunk, first);
@@ -313,7 +332,8 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const float* __restr
   if (tid < hd) {
     float total = 0.f;
     for (int g = 0; g < groups; ++g) total += sm_part[g * hd + tid];
-    const float l = ((sm_sum[0] + sm_sum[1]) + sm_sum[2]) + sm_sum[3];
+    float l = ((sm_sum[0] + sm_sum[1]) + sm_sum[2]) + sm_sum[3];
+    if (ex.sinks) l += __expf(ex.sinks[head] - top);
     store_out(out + (size_t)s * out_stride + (size_t)head * hd + tid, total / l);
   }
 }
@@ -402,7 +422,7 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
                                              const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[T][HD / 16],
                                              bf16x8 (&vf)[(HD + 31) / 32][2 * T], const PageSource& src, int kbase, int next,
                                              const int (&lo)[QB], const int (&hi)[QB], bool mask, float c, int lane,
-                                             int keep = 0) {
+                                             int keep = 0, float cap_in = 0.f, float cap_out = 0.f) {
   constexpr int KS = HD / 16, DB = (HD + 31) / 32;
   constexpr int LAST = (ACT & 2) ? 1 : 0;
   const int g = lane >> 5;
@@ -426,6 +446,12 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
       // not earlier: above the score products the old and the new fragments would both need registers
       __builtin_amdgcn_sched_barrier(0);
       load_keys<HD, T>(kf, src, next, lane);
+    }
+    if (cap_in > 0.f) {  // capped scores, kept in the raw scores' unit (the same for the whole wave)
+#pragma unroll
+      for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[t][r] = cap_out * tanh_fast(s[t][r] * cap_in);
     }
     if (mask) {  // the same for the whole wave
 #pragma unroll
@@ -490,14 +516,14 @@ struct BlockRange {
   __device__ bool unmasked(int kb, int span = 64) const { return whole && kb >= free_lo && kb + span - 1 <= free_hi; }
 };
 
-__device__ __forceinline__ BlockRange block_range(int t0, int qlen, int p0, int window) {
+__device__ __forceinline__ BlockRange block_range(int t0, int qlen, int p0, int window, int span = 0) {
   BlockRange r;
   const int t1 = min(t0 + 32, qlen) - 1;
   r.whole = t0 + 32 <= qlen;
   r.last = p0 + t1;
-  r.first = window > 0 ? max(0, p0 + t0 - window + 1) : 0;
+  r.first = first_key(p0 + t0, window, span);
   r.free_hi = p0 + t0;
-  r.free_lo = window > 0 ? max(0, p0 + t1 - window + 1) : 0;
+  r.free_lo = first_key(p0 + t1, window, span);
   return r;
 }
 
@@ -544,7 +570,8 @@ __device__ __forceinline__ void store_part(const f32x16 (&acc)[(HD + 31) / 32], 
 // Adds the parts in their order: one workgroup of HD threads per (row, head).
 template <typename OT>
 __global__ void prefill_parts_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, OT* __restrict__ out,
-                                     int out_stride, int first_row, int n_rows, int nh, int hd, int parts, float c) {
+                                     int out_stride, int first_row, int n_rows, int nh, int hd, int parts, float c,
+                                     const float* __restrict__ sinks) {
   const int row = blockIdx.x / nh, head = blockIdx.x % nh, d = threadIdx.x;
   if (d >= hd) return;
   const size_t cell = (size_t)row * nh + head, stride = (size_t)n_rows * nh;
@@ -557,6 +584,7 @@ __global__ void prefill_parts_kernel(const float* __restrict__ part_acc, const f
     val += part_acc[(k * stride + cell) * hd + d] * f;
     l += part_ml[(k * stride + cell) * 2 + 1] * f;
   }
+  if (sinks) l += __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - top * c);
   store_out(out + (size_t)(first_row + row) * out_stride + (size_t)head * hd + d, val / l);
 }
 
@@ -612,7 +640,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
                                                       const bf16* __restrict__ kp, const bf16* __restrict__ vp, int nh, int nkv,
                                                       int page_shift, float scale, int window, int keep,
                                                       float* __restrict__ part_acc, float* __restrict__ part_ml, int parts,
-                                                      int first_row, int n_rows) {
+                                                      int first_row, int n_rows, Extra ex) {
   // parts > 1: `parts` workgroups share a group's pairs, taking the tiles of keys in turn like the waves of a pair
   // do; each writes its sums to part_acc / part_ml (rows counted from first_row), and prefill_parts_kernel adds them.
   constexpr bool WIDE = std::is_same<OT, float>::value;   // results that go on in 32-bit: weights in two parts
@@ -643,6 +671,9 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
   PageSource src{kp, vp, tables + (size_t)seq * table_stride, nkv, kvh, page_shift, 0, 0, (keep + 15) & ~15};
   const size_t row0 = (size_t)q_start[seq];
   const float c = scale * 1.4426950408889634f;
+  const float cap_in = ex.softcap > 0.f ? scale / ex.softcap : 0.f, cap_out = ex.softcap > 0.f ? ex.softcap / scale : 0.f;
+  // a sink's share of a token's denominator, given the token's running maximum (in the raw scores' unit)
+  auto sink_of = [&](float m) { return ex.sinks ? __builtin_amdgcn_exp2f(ex.sinks[head] * 1.4426950408889634f - m * c) : 0.f; };
   constexpr int T = QB == 2 ? 2 : 1;  // tiles of 32 keys a step: with one block live at a time (the larger head
                                       // sizes) the fragments of 64 keys would not fit the registers
   bf16x8 kf[T][KS];
@@ -668,7 +699,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       const int tok = start[qb] + col;
       const bool valid = works && tok < qlen && (qb == 0 || has_second);
       const int p = p0 + tok;
-      lo[qb] = valid ? (window > 0 ? max(0, p - window + 1) : 0) : 1;
+      lo[qb] = valid ? first_key(p, window, ex.span) : 1;
       hi[qb] = valid ? p : 0;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
@@ -679,7 +710,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[qb][b][r] = 0.f;
-      range[qb] = block_range(start[qb], qlen, p0, window);
+      range[qb] = block_range(start[qb], qlen, p0, window, ex.span);
     }
     const int end = has_second ? range[1].last : range[0].last;
     src.tlo = range[0].first & ~15;
@@ -707,18 +738,18 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       while (kb <= range[0].last) {
         const int next = my_next(kb);
         const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));
-        attend64_q32<HD, 2, 3, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep);
+        attend64_q32<HD, 2, 3, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep, cap_in, cap_out);
         kb = next;
       }
       while (kb <= range[1].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 2, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep);
+        attend64_q32<HD, 2, 2, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep, cap_in, cap_out);
         kb = next;
       }
     } else {
       while (kb <= range[0].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 1, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep);
+        attend64_q32<HD, 2, 1, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep, cap_in, cap_out);
         kb = next;
       }
     }
@@ -738,14 +769,14 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
         store_part<HD>(acc[qb], m[qb], total, part_acc + cell * HD, part_ml + cell * 2, g);
         continue;
       }
-      store_block<HD, OT>(acc[qb], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+      store_block<HD, OT>(acc[qb], total + sink_of(m[qb]), out + (row0 + tok) * out_stride + (size_t)head * HD, g);
     }
   } else {
     for (int which = 0; which < (has_second ? 2 : 1); ++which) {
       const int tok = start[which] + col;
       const bool valid = tok < qlen;
       const int p = p0 + tok;
-      int lo[1] = {valid ? (window > 0 ? max(0, p - window + 1) : 0) : 1}, hi[1] = {valid ? p : 0};
+      int lo[1] = {valid ? first_key(p, window, ex.span) : 1}, hi[1] = {valid ? p : 0};
       float m[1] = {-INFINITY}, l[1] = {0.f};
       f32x16 acc[1][DB];
 #pragma unroll
@@ -755,7 +786,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       for (int b = 0; b < DB; ++b)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[0][b][r] = 0.f;
-      const BlockRange range = block_range(start[which], qlen, p0, window);
+      const BlockRange range = block_range(start[which], qlen, p0, window, ex.span);
       src.tlo = range.first & ~15;
       src.thi = range.last & ~15;
       constexpr int SPAN = 32 * T;  // the waves of the pair take the steps of SPAN keys in turn
@@ -768,7 +799,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       load_values<HD, T>(vf, src, key_of(i0), lane);
       for (int i = i0; key_of(i) <= range.last; i += stride)
         attend64_q32<HD, 1, 1, T, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, key_of(i), key_of(i + stride), lo, hi,
-                                  !range.unmasked(key_of(i), SPAN), c, lane, keep);
+                                  !range.unmasked(key_of(i), SPAN), c, lane, keep, cap_in, cap_out);
       if constexpr (SPLIT > 1) {
         hand_over<DB, SPLIT>(m[0], l[0], acc[0], handed[wave], handed_ml[wave], half, lane, c, which > 0);
         if (half != 0) continue;
@@ -778,7 +809,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
         const size_t cell = ((size_t)part * n_rows + (row0 + tok - first_row)) * nh + head;
         store_part<HD>(acc[0], m[0], total, part_acc + cell * HD, part_ml + cell * 2, g);
       } else if (valid) {
-        store_block<HD, OT>(acc[0], total, out + (row0 + tok) * out_stride + (size_t)head * HD, g);
+        store_block<HD, OT>(acc[0], total + sink_of(m[0]), out + (row0 + tok) * out_stride + (size_t)head * HD, g);
       }
     }
   }
@@ -797,8 +828,9 @@ template <typename OT>
 static int decode_launch(const void* q, int q_stride, OT* out, int out_stride, void* ws_acc, void* ws_ml,
                          const int32_t* positions, const int32_t* tables, int table_stride, const void* k_pages,
                          const void* v_pages, int n_decode, int nh, int nkv, int hd, int page_size, float scale, int window,
-                         int keep_first, int chunk, int max_context, hipStream_t stream) {
+                         int keep_first, int chunk, int max_context, hipStream_t stream, Extra ex = Extra{0, 0.f, nullptr}) {
   GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_decode: kept first keys go with a window");
+  GB_REQUIRE(ex.span >= 0 && (ex.span == 0 || window == 0) && ex.softcap >= 0.f, "attention_decode: runs of positions exclude a window; a cap is positive or 0");
   GB_REQUIRE(n_decode >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_decode: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_decode: head size %d is not a multiple of 16 up to 128", hd);
   GB_REQUIRE(nh / nkv <= 16, "attention_decode: %d query heads per kv head exceed the 16 columns of a tile", nh / nkv);
@@ -823,11 +855,11 @@ static int decode_launch(const void* q, int q_stride, OT* out, int out_stride, v
     if (waves == 16)                                                                                                        \
       hipLaunchKernelGGL((decode_kernel<HD, 16, OT>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride, \
                          (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
-                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits);                           \
+                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits, ex);                       \
     else                                                                                                                    \
       hipLaunchKernelGGL((decode_kernel<HD, 4, OT>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride,  \
                          (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
-                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits);                           \
+                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits, ex);                       \
   }
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
@@ -835,7 +867,7 @@ static int decode_launch(const void* q, int q_stride, OT* out, int out_stride, v
   if (splits > 1) {
     GB_REQUIRE(splits <= 256, "attention_decode: %d chunks are more than the 256 the second pass combines", splits);
     hipLaunchKernelGGL(decode_reduce_kernel<OT>, dim3(n_decode * nh), dim3(256), 0, stream, (const float*)ws_acc,
-                       (const float*)ws_ml, out, out_stride, positions, nh, hd, window, keep_first, chunk, splits);
+                       (const float*)ws_ml, out, out_stride, positions, nh, hd, window, keep_first, chunk, splits, ex);
     return launched("attention_decode_reduce");
   }
   return 0;
@@ -970,8 +1002,9 @@ static int prefill_launch(const void* q, int q_stride, OT* out, int out_stride, 
                           const int32_t* pos0, int seq_base, int n_seqs, int max_q_len, int max_context, const int32_t* tables,
                           int table_stride, const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
                           float scale, int window, int keep_first, int first_row, int n_rows, float* part_ws,
-                          long long part_floats, hipStream_t stream) {
+                          long long part_floats, hipStream_t stream, Extra ex = Extra{0, 0.f, nullptr}) {
   GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_prefill: kept first keys go with a window");
+  GB_REQUIRE(ex.span >= 0 && (ex.span == 0 || window == 0) && ex.softcap >= 0.f, "attention_prefill: runs of positions exclude a window; a cap is positive or 0");
   GB_REQUIRE(n_seqs >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad head counts nh=%d nkv=%d", nh, nkv);
   GB_REQUIRE(gb_attention_supported_head_size(hd), "attention_prefill: head size %d is not a multiple of 16 up to 128", hd);
   GB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0, "attention_prefill: page size %d is not a power of two from 16 up", page_size);
@@ -997,7 +1030,7 @@ static int prefill_launch(const void* q, int q_stride, OT* out, int out_stride, 
   hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT, OT>), grid, block, 0, stream, (const bf16*)q, q_stride, out, \
                      out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages,               \
                      (const bf16*)v_pages, nh, nkv, page_shift, scale, window, keep_first, part_acc, part_ml, parts, first_row, \
-                     n_rows)
+                     n_rows, ex)
 #define GB_CASE(HD)                                        \
   if (hd == HD) {                                          \
     if constexpr (HD <= 64) {                              \
@@ -1017,7 +1050,7 @@ static int prefill_launch(const void* q, int q_stride, OT* out, int out_stride, 
   if (int rc = launched("attention_prefill")) return rc;
   if (parts > 1) {
     hipLaunchKernelGGL(prefill_parts_kernel<OT>, dim3((unsigned)(n_rows * nh)), dim3((hd + 63) / 64 * 64), 0, stream, part_acc,
-                       part_ml, out, out_stride, first_row, n_rows, nh, hd, parts, scale * 1.4426950408889634f);
+                       part_ml, out, out_stride, first_row, n_rows, nh, hd, parts, scale * 1.4426950408889634f, ex.sinks);
     return launched("attention_prefill (second pass)");
   }
   return 0;
@@ -1058,7 +1091,45 @@ extern "C" int gb_attention_prefill_bf16(const void* q, int q_stride, void* out,
                                         window, 0, first_row, n_rows, part_ws, part_floats, stream);
 }
 
+// The same two with everything a mixer may ask of the softmax: a window with kept first keys, or runs of `span`
+// positions; capped scores; sinks [nh] (see Extra).  out32 != 0: float32 result rows.
+extern "C" int gb_attention_decode_bf16_by(const void* q, int q_stride, void* out, int out_stride, int out32, void* ws_acc,
+                                           void* ws_ml, const int32_t* positions, const int32_t* tables, int table_stride,
+                                           const void* k_pages, const void* v_pages, int n_decode, int nh, int nkv, int hd,
+                                           int page_size, float scale, int window, int keep_first, int span, float softcap,
+                                           const float* sinks, int chunk, int max_context, hipStream_t stream) {
+  const Extra ex{span, softcap, sinks};
+  if (out32) {
+    GB_REQUIRE((uintptr_t)out % 16 == 0, "attention_decode: float32 result rows must be 16-byte aligned");
+    return decode_launch<float>(q, q_stride, (float*)out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k_pages,
+                                v_pages, n_decode, nh, nkv, hd, page_size, scale, window, keep_first, chunk, max_context, stream, ex);
+  }
+  return decode_launch<bf16>(q, q_stride, (bf16*)out, out_stride, ws_acc, ws_ml, positions, tables, table_stride, k_pages, v_pages,
+                             n_decode, nh, nkv, hd, page_size, scale, window, keep_first, chunk, max_context, stream, ex);
+}
+
+extern "C" int gb_attention_prefill_bf16_by(const void* q, int q_stride, void* out, int out_stride, int out32,
+                                            const int32_t* q_start, const int32_t* q_len, const int32_t* pos0, int seq_base,
+                                            int n_seqs, int max_q_len, int max_context, const int32_t* tables, int table_stride,
+                                            const void* k_pages, const void* v_pages, int nh, int nkv, int hd, int page_size,
+                                            float scale, int window, int keep_first, int span, float softcap,
+                                            const float* sinks, int first_row, int n_rows, float* part_ws,
+                                            long long part_floats, hipStream_t stream) {
+  const Extra ex{span, softcap, sinks};
+  if (out32) {
+    GB_REQUIRE((uintptr_t)out % 16 == 0, "attention_prefill: float32 result rows must be 16-byte aligned");
+    return prefill_launch<float>(q, q_stride, (float*)out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len,
+                                 max_context, tables, table_stride, k_pages, v_pages, nh, nkv, hd, page_size, scale, window,
+                                 keep_first, first_row, n_rows, part_ws, part_floats, stream, ex);
+  }
+  return prefill_launch<bf16>(q, q_stride, (bf16*)out, out_stride, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, max_context,
+                              tables, table_stride, k_pages, v_pages, nh, nkv, hd, page_size, scale, window, keep_first, first_row,
+                              n_rows, part_ws, part_floats, stream, ex);
+}
+
 // the launches of a layer can be recorded and made again for the layers like it (common.h)
+GB_TAPED(gb_attention_decode_bf16_by)
+GB_TAPED(gb_attention_prefill_bf16_by)
 GB_TAPED(gb_attention_decode_bf16_keep)
 GB_TAPED(gb_attention_prefill_bf16_keep)
 GB_TAPED(gb_attention_decode_bf16_out32)

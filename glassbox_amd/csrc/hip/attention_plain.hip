@@ -6,6 +6,9 @@
 // Token t of request s at position p reads keys lo..p of its own request through the block
 // table, lo = 0 or p - window + 1 (crates/glassbox-core/src/model.rs:285-312):
 //   score = dot(q, k) * scale ; prob = softmax(score) ; out = sum prob * v
+// Options: `span` > 0: positions are cut into runs of `span` from 0 on and lo is the first position of p's run (a token
+// sees its own run only); `softcap` > 0: score = softcap * tanh(score / softcap); `sinks`: one number a query head whose
+// exponential joins the softmax's denominator and which has no value (the weights then sum to less than one).
 //
 // The order of every addition depends on the token's position alone, not on the batch and not
 // on how the work is spread over workgroups.  Keys go in chunks of 256 from lo on.  A chunk is
@@ -93,6 +96,13 @@ struct Shape {
   int nh, nkv, hd, page_size, window, table_stride;
   float scale;
   int keep;   // with a window: keys 0 .. keep - 1 stay visible to every later token
+  int span;   // > 0: a token sees the keys of its own run of `span` positions (runs counted from position 0)
+  float softcap;        // > 0: scores pass softcap * tanh(score / softcap)
+  const float* sinks;   // [nh] or null: exp(sinks[h]) is added to the softmax's denominator of head h
+  __device__ __forceinline__ float score(float dot) const {
+    const float s = dot * scale;
+    return softcap > 0.f ? softcap * tanhf(s / softcap) : s;
+  }
 };
 
 // The chunks of the token at position pos.  Without kept first keys: from lo = the window's first key (or 0) on.
@@ -101,7 +111,7 @@ struct Shape {
 struct Chunks {
   int lo, kept, n_kept, n;
   __device__ __forceinline__ Chunks(const Shape& sh, int pos) {
-    lo = sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
+    lo = sh.span > 0 ? pos - pos % sh.span : sh.window > 0 ? max(0, pos - sh.window + 1) : 0;
     kept = sh.keep > 0 ? min(sh.keep, lo) : 0;
     n_kept = (kept + kChunk - 1) / kChunk;
     n = n_kept + (pos - lo) / kChunk + 1;
@@ -126,7 +136,7 @@ __device__ __forceinline__ void chunk_alone(const Shape& sh, const float* qs, fl
   if (p <= hi) {
     const int page = table[p / ps];
     const T* kb = k_pages + ((size_t)page * sh.nkv + kvh) * ps * hd;
-    s = key_dot<T>(qs, kb, p % ps, hd, ps, key_piece(hd)) * sh.scale;
+    s = sh.score(key_dot<T>(qs, kb, p % ps, hd, ps, key_piece(hd)));
   }
   m_c = block_max(s, scratch);
   const float e = p <= hi ? expf(s - m_c) : 0.f;
@@ -160,8 +170,9 @@ __device__ __forceinline__ void chunk_alone(const Shape& sh, const float* qs, fl
 
 // The end: a dimension's words added in ascending order, divided by the sum.
 template <typename T, int PER>
-__device__ __forceinline__ void finish(const Shape& sh, float* comb, const float (&acc)[PER], float l, T* out_row) {
+__device__ __forceinline__ void finish(const Shape& sh, float* comb, const float (&acc)[PER], const Running& r, int h, T* out_row) {
   const int tid = threadIdx.x;
+  const float l = sh.sinks ? r.l + expf(sh.sinks[h] - r.m) : r.l;
   const int words = sh.page_size / 4, pairs = sh.hd * words;
 #pragma unroll
   for (int u = 0; u < PER; ++u) {
@@ -223,7 +234,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_kernel(
     chunk_alone<T, PER>(sh, qs, es, scratch, table, k_pages, v_pages, kvh, c0, ch.last(c, pos), m_c, l_c, a_c);
     merge_chunk<PER>(r, acc, m_c, l_c, a_c);
   }
-  finish<T, PER>(sh, comb, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
+  finish<T, PER>(sh, comb, acc, r, h, out + (size_t)t * out_stride + (size_t)h * sh.hd);
 }
 
 // ---- several tokens a workgroup ------------------------------------------------------------------------------
@@ -315,7 +326,7 @@ __device__ __forceinline__ void chunk_together(const Shape& sh, const T* __restr
     key_dots<T, Q>(q0, q_stride, kb, p % ps, hd, ps, key_piece(hd), dot);
 #pragma unroll
     for (int j = 0; j < Q; ++j)
-      if (p <= hi[j]) s[j] = dot[j] * sh.scale;
+      if (p <= hi[j]) s[j] = sh.score(dot[j]);
   }
 #pragma unroll
   for (int j = 0; j < Q; ++j) m_c[j] = s[j];
@@ -387,7 +398,7 @@ __device__ __forceinline__ void walk_together(const Shape& sh, const T* __restri
   }
 #pragma unroll
   for (int j = 0; j < Q; ++j) {
-    finish<T, PER>(sh, comb, acc[j], r[j].l, out + (size_t)(first + j) * out_stride + (size_t)h * sh.hd);
+    finish<T, PER>(sh, comb, acc[j], r[j], h, out + (size_t)(first + j) * out_stride + (size_t)h * sh.hd);
     __syncthreads();   // comb is written again for the next token
   }
 }
@@ -407,7 +418,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_group_kernel(
   const int first = g * kGroup, count = min(kGroup, n - first);
   const int tid = threadIdx.x;
   const int pos0 = positions[first], seq0 = tok_seq[first];
-  bool together = count == kGroup && sh.window == 0;
+  bool together = count == kGroup && sh.window == 0 && sh.span == 0;
   for (int j = 1; j < count; ++j) together = together && tok_seq[first + j] == seq0 && positions[first + j] == pos0 + j;
 
   if (together) {
@@ -437,7 +448,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_group_kernel(
                           ch.last(c, pos), m_c, l_c, a_c);
       merge_chunk<PER>(r, acc, m_c, l_c, a_c);
     }
-    finish<T, PER>(sh, comb, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
+    finish<T, PER>(sh, comb, acc, r, h, out + (size_t)t * out_stride + (size_t)h * sh.hd);
     __syncthreads();   // comb is written again for the next token
   }
 }
@@ -463,7 +474,7 @@ __global__ __launch_bounds__(kChunk) void attention_plain_merge_kernel(T* __rest
     for (int u = 0; u < PER; ++u) a_c[u] = cell[u * kChunk + tid];
     merge_chunk<PER>(r, acc, cell[PER * kChunk], cell[PER * kChunk + 1], a_c);
   }
-  finish<T, PER>(sh, smem, acc, r.l, out + (size_t)t * out_stride + (size_t)h * sh.hd);
+  finish<T, PER>(sh, smem, acc, r, h, out + (size_t)t * out_stride + (size_t)h * sh.hd);
 }
 
 inline int own_pairs(int hd, int page_size) {
@@ -485,7 +496,7 @@ void launch(const void* q, int q_stride, void* out, int out_stride, const int32_
                        (const T*)k_pages, (const T*)v_pages, sh, ws, max_chunks);
     hipLaunchKernelGGL((attention_plain_merge_kernel<T, PER>), dim3((unsigned)(n * sh.nh)), dim3(kChunk), comb, stream,
                        (T*)out, out_stride, positions, sh, (const float*)ws, max_chunks);
-  } else if (grouped_form && PER <= kGroupMaxOwn && sh.window == 0) {   // (elsewhere the one-token form: the same bits)
+  } else if (grouped_form && PER <= kGroupMaxOwn && sh.window == 0 && sh.span == 0) {   // (elsewhere the one-token form: the same bits)
     if constexpr (PER <= kGroupMaxOwn) {
       const size_t grouped = sizeof(float) * (kGroup * (sh.hd + kChunk + 4) + 17) + comb;
       const int groups = (n + kGroup - 1) / kGroup;
@@ -537,14 +548,17 @@ extern "C" long long gb_attention_plain_split_floats(int n, int nh, int hd, int 
 extern "C" int gb_attention_plain(const void* q, int q_stride, void* out, int out_stride, int dtype,
                                   const int32_t* positions, const int32_t* tok_seq, const int32_t* tables,
                                   int table_stride, const void* k_pages, const void* v_pages, int n, int nh, int nkv,
-                                  int hd, int page_size, float scale, int window, int keep_first, float* ws,
-                                  long long ws_floats, int max_context, int grouped, hipStream_t stream) {
+                                  int hd, int page_size, float scale, int window, int keep_first, int span,
+                                  float softcap, const float* sinks, float* ws, long long ws_floats, int max_context,
+                                  int grouped, hipStream_t stream) {
   GB_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_plain: bad sizes n=%d nh=%d nkv=%d hd=%d", n, nh, nkv, hd);
   GB_REQUIRE(nh % nkv == 0, "attention_plain: %d query heads are not a multiple of %d key heads", nh, nkv);
   GB_REQUIRE(hd <= kChunk, "attention_plain: head size %d is above the supported 256", hd);
   GB_REQUIRE(q_stride >= nh * hd && out_stride >= nh * hd, "attention_plain: row strides shorter than the heads");
   GB_REQUIRE(page_size > 0 && table_stride > 0 && window >= 0, "attention_plain: bad page size, table stride or window");
   GB_REQUIRE(keep_first >= 0 && (keep_first == 0 || window > 0), "attention_plain: kept first keys go with a window");
+  GB_REQUIRE(span >= 0 && (span == 0 || window == 0), "attention_plain: runs of positions and a window exclude each other");
+  GB_REQUIRE(softcap >= 0.f, "attention_plain: a cap of the scores is positive, or 0 for none");
   GB_REQUIRE(page_size % 4 == 0, "attention_plain: a page of %d tokens is not whole words of four slots", page_size);
   GB_REQUIRE((long long)n * nh < (1ll << 31), "attention_plain: too many (token, head) pairs");
   const int per = own_pairs(hd, page_size);
@@ -561,7 +575,7 @@ extern "C" int gb_attention_plain(const void* q, int q_stride, void* out, int ou
                "attention_plain: the workspace holds %lld floats, %lld are needed", ws_floats,
                gb_attention_plain_split_floats(n, nh, hd, page_size, max_context, keep_first));
   }
-  const Shape sh{nh, nkv, hd, page_size, window, table_stride, scale, keep_first};
+  const Shape sh{nh, nkv, hd, page_size, window, table_stride, scale, keep_first, span, softcap, sinks};
   if (dtype == kF32)
     return launch_by_pairs<float>(per, q, q_stride, out, out_stride, positions, tok_seq, tables, k_pages, v_pages, n, sh, ws,
                                   max_chunks, grouped != 0, stream);

@@ -4,6 +4,11 @@
 //   chosen: the `top` experts with the largest s + correction (of equal ones the lower index)
 //   weight of a chosen expert: s / (sum of the chosen s + 1e-20) * scale
 //
+// Other routers are the same kernel with other arguments: scores by softmax over all experts instead of the sigmoid;
+// weights that are the scores as they stand (times scale), not divided by their sum; experts in `groups` equal runs
+// of neighbours, of which only the `keep` runs with the largest pick score (s + correction) of any of their experts can
+// be chosen; a shared expert that counts fully (weight 1) instead of through a gate of its own.
+//
 // `route` leaves the result in two forms: the chosen experts and their weights a token ([n, top]), and a row of E
 // weights a token with zeros for the experts not chosen (with `shared`, one more column: sigmoid of z's column E, the
 // gate of an expert that every token uses).  `gated_units` turns the stacked gate and up projections of all experts
@@ -28,22 +33,69 @@ namespace {
 constexpr int kPerLane = 8;   // experts a lane: up to 512 experts
 constexpr int kMaxTop = 16;
 
+// shared: 0 none, 1 a gate sigmoid(z[E]), 2 weight 1.  softmax: scores over all experts (else sigmoid of each).
+// renorm: weights divided by the sum of the chosen scores.  groups > 0: see above.
 __global__ __launch_bounds__(4 * kWave) void route_kernel(const float* __restrict__ z, int ldz, int E,
                                                         const float* __restrict__ correction, int top, float scale,
-                                                        int shared, float* __restrict__ combine, int32_t* __restrict__ ids,
+                                                        int shared, int softmax, int renorm, int groups, int keep,
+                                                        float* __restrict__ combine, int32_t* __restrict__ ids,
                                                         float* __restrict__ wts, int n) {
-  const int t = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  if (t >= n) return;
+  __shared__ float pick[4][kPerLane * kWave];   // a wave's pick scores, for the groups' maxima
+  __shared__ float best_of[4][kWave];           // a group's best pick score, then 1 if the group is kept
+  const int wave = threadIdx.x / kWave;
+  const int t = blockIdx.x * 4 + wave, lane = threadIdx.x % kWave;
+  if (t >= n) return;   // (a wave as a whole: no barrier below, a wave's lanes run together)
   const float* row = z + (size_t)t * ldz;
   float s[kPerLane], c[kPerLane];
+  float top_z = -INFINITY, denom = 0.f;
+  if (softmax) {
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j)
+      if (lane + j * kWave < E) top_z = fmaxf(top_z, row[lane + j * kWave]);
+    top_z = wave_max(top_z);
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j)
+      if (lane + j * kWave < E) denom += expf(row[lane + j * kWave] - top_z);
+    denom = wave_sum(denom);
+  }
 #pragma unroll
   for (int j = 0; j < kPerLane; ++j) {
     const int e = lane + j * kWave;
     s[j] = 0.f;
     c[j] = -INFINITY;
     if (e < E) {
-      s[j] = 1.0f / (1.0f + expf(-row[e]));
+      s[j] = softmax ? expf(row[e] - top_z) / denom : 1.0f / (1.0f + expf(-row[e]));
       c[j] = s[j] + (correction ? correction[e] : 0.f);
+    }
+  }
+  if (groups > 0) {
+    const int size = E / groups;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j)
+      if (lane + j * kWave < E) pick[wave][lane + j * kWave] = c[j];
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    float mine = -INFINITY;   // lane g: group g's best
+    if (lane < groups)
+      for (int i = 0; i < size; ++i) mine = fmaxf(mine, pick[wave][lane * size + i]);
+    best_of[wave][lane] = mine;
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    int ahead = 0;            // groups that go before this one: a larger best, or the same and a lower number
+    if (lane < groups)
+      for (int g = 0; g < groups; ++g) {
+        const float o = best_of[wave][g];
+        ahead += (o > mine || (o == mine && g < lane)) ? 1 : 0;
+      }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    best_of[wave][lane] = (lane < groups && ahead < keep) ? 1.f : 0.f;
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+      const int e = lane + j * kWave;
+      if (e < E && best_of[wave][e / size] == 0.f) c[j] = -INFINITY;
     }
   }
   int chosen[kMaxTop];
@@ -83,7 +135,7 @@ __global__ __launch_bounds__(4 * kWave) void route_kernel(const float* __restric
     for (int j = 0; j < kPerLane; ++j)
       if (lane + j * kWave == be) c[j] = -INFINITY;   // taken
   }
-  const float inv = scale / (sum + 1e-20f);
+  const float inv = renorm ? scale / (sum + 1e-20f) : scale;
   const int cols = E + (shared ? 1 : 0);
 #pragma unroll
   for (int j = 0; j < kPerLane; ++j) {
@@ -95,7 +147,7 @@ __global__ __launch_bounds__(4 * kWave) void route_kernel(const float* __restric
       if (k < top && chosen[k] == e) w = cs[k] * inv;
     combine[(size_t)t * cols + e] = w;
   }
-  if (shared && lane == 0) combine[(size_t)t * cols + E] = 1.0f / (1.0f + expf(-row[E]));
+  if (shared && lane == 0) combine[(size_t)t * cols + E] = shared == 2 ? 1.0f : 1.0f / (1.0f + expf(-row[E]));
 #pragma unroll
   for (int k = 0; k < kMaxTop; ++k)
     if (k < top && lane == k % kWave) {
@@ -125,6 +177,24 @@ __global__ void gated_units_kernel(const I* __restrict__ gu, int ld, const float
     y = g / (1.0f + expf(-g)) * u * w;
   }
   act[idx] = from_f<O>(y);
+}
+
+// act[t, j] = relu(z[t, j])^2 * combine[t, expert of column j] for units without a gate half: columns
+// e * ff .. (e + 1) * ff - 1 are expert e's, those from E * ff on the shared expert's.  Without `combine` every weight is 1.
+template <typename I, typename O>
+__global__ void relu2_units_kernel(const I* __restrict__ z, int ld, const float* __restrict__ combine, int cols, O* __restrict__ act,
+                                   int lda, long long count, int inter, int E, int ff) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= count) return;
+  const long long t = idx / inter;
+  const int j = (int)(idx % inter);
+  const float w = combine ? combine[(size_t)t * cols + (j < E * ff ? j / ff : E)] : 1.f;
+  float y = 0.f;
+  if (w != 0.f) {
+    const float v = fmaxf(to_f(z[(size_t)t * ld + j]), 0.f);
+    y = v * v * w;
+  }
+  act[(size_t)t * lda + j] = from_f<O>(y);
 }
 
 // counts[e]: how many of the n * top entries chose expert e.  One workgroup an expert.
@@ -238,15 +308,44 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
 
 }  // namespace
 
-extern "C" int gb_moe_route(const float* z, int ldz, int n, int E, const float* correction, int top, float scale, int shared,
-                            float* combine, int32_t* ids, float* wts, hipStream_t stream) {
+extern "C" int gb_moe_route_by(const float* z, int ldz, int n, int E, const float* correction, int top, float scale, int shared,
+                               int softmax, int renorm, int groups, int keep, float* combine, int32_t* ids, float* wts,
+                               hipStream_t stream) {
   GB_REQUIRE(n >= 0 && E > 0 && E <= kPerLane * kWave, "moe_route: %d experts (at most %d)", E, kPerLane * kWave);
   GB_REQUIRE(top > 0 && top <= kMaxTop && top <= E, "moe_route: %d chosen experts of %d (at most %d)", top, E, kMaxTop);
-  GB_REQUIRE(ldz >= E + (shared ? 1 : 0), "moe_route: rows of %d logits for %d experts", ldz, E);
+  GB_REQUIRE(shared >= 0 && shared <= 2 && ldz >= E + (shared == 1 ? 1 : 0), "moe_route: rows of %d logits for %d experts", ldz, E);
+  GB_REQUIRE(groups >= 0 && (groups == 0 || (groups <= kWave && E % groups == 0 && keep >= 1 && keep <= groups &&
+                                             keep * (E / groups) >= top)),
+             "moe_route: %d groups of %d experts, %d kept, %d experts a token", groups, E, keep, top);
   if (n == 0) return 0;
   hipLaunchKernelGGL(route_kernel, dim3((unsigned)((n + 3) / 4)), dim3(4 * kWave), 0, stream, z, ldz, E, correction, top, scale,
-                     shared, combine, ids, wts, n);
+                     shared, softmax, renorm, groups, keep, combine, ids, wts, n);
   return launched("moe_route");
+}
+
+extern "C" int gb_moe_route(const float* z, int ldz, int n, int E, const float* correction, int top, float scale, int shared,
+                            float* combine, int32_t* ids, float* wts, hipStream_t stream) {
+  return gb_moe_route_by(z, ldz, n, E, correction, top, scale, shared ? 1 : 0, 0, 1, 0, 0, combine, ids, wts, stream);
+}
+
+extern "C" int gb_moe_relu2_units(const void* z, int in_dtype, int ld, const float* combine, int cols, void* act, int out_dtype,
+                                  int lda, int n, int inter, int E, int ff, hipStream_t stream) {
+  GB_REQUIRE(n >= 0 && inter > 0 && ld >= inter && lda >= inter && E >= 0 && ff > 0 && E * ff <= inter &&
+                 (!combine || cols >= E + (E * ff < inter ? 1 : 0)),
+             "moe_relu2_units: bad sizes n=%d inter=%d experts=%d of %d cols=%d", n, inter, E, ff, cols);
+  if (n == 0) return 0;
+  const long long count = (long long)n * inter;
+  GB_REQUIRE((count + 255) / 256 < (1ll << 31), "moe_relu2_units: too many elements");
+  const dim3 grid((unsigned)((count + 255) / 256));
+  if (in_dtype == kF32 && out_dtype == kF32)
+    hipLaunchKernelGGL((relu2_units_kernel<float, float>), grid, dim3(256), 0, stream, (const float*)z, ld, combine, cols, (float*)act, lda, count, inter, E, ff);
+  else if (in_dtype == kF32 && out_dtype == kBF16)
+    hipLaunchKernelGGL((relu2_units_kernel<float, bf16>), grid, dim3(256), 0, stream, (const float*)z, ld, combine, cols, (bf16*)act, lda, count, inter, E, ff);
+  else if (in_dtype == kBF16 && out_dtype == kBF16)
+    hipLaunchKernelGGL((relu2_units_kernel<bf16, bf16>), grid, dim3(256), 0, stream, (const bf16*)z, ld, combine, cols, (bf16*)act, lda, count, inter, E, ff);
+  else
+    return fail("moe_relu2_units: no kernel for operand type %d and result type %d", in_dtype, out_dtype);
+  return launched("moe_relu2_units");
 }
 
 extern "C" int gb_moe_gated_units(const void* gu, int in_dtype, int ld, const float* combine, int cols, void* act, int out_dtype,
@@ -299,4 +398,6 @@ extern "C" int gb_moe_combine(const float* y, int ldy, const int32_t* pos, const
 GB_TAPED(gb_moe_sort)
 GB_TAPED(gb_moe_combine)
 GB_TAPED(gb_moe_route)
+GB_TAPED(gb_moe_route_by)
+GB_TAPED(gb_moe_relu2_units)
 GB_TAPED(gb_moe_gated_units)

@@ -89,8 +89,27 @@ _SIGS = {
         # x, y, slices, slice stride, g, eps, rounded, dtype, n, d, conv w, taps, state, tok_seq, pos0, state slots, stream
         "gb_norm_add": [_vp, _vp, _i, C.c_longlong, _vp, _f, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp],
     },
+    "tanhmix": {
+        # x, ldx, rows, alpha, w, b, out, its dtype, ldo, n, d, stream
+        "gb_tanh_norm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+        # x, y, slices, slice stride, alpha, w, b, next alpha, w, b, h, its dtype, n, d, stream
+        "gb_tanh_norm_add": [_vp, _vp, _i, C.c_longlong, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+        # proj, dtype, ld, bias, wconv, taps, state, tok_seq, q_start, pos0, state slots, single, wq, wk, eps, joint, cos, sin,
+        # rot, mag, neighbours, tied, out, ldo, hd, slots, k, v, page, n, H, G, dk, dv, stream
+        "gb_qk_heads": [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _f, _i, _vp, _vp, _i, _f, _i, _i, _vp, _i,
+                        _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+        # proj, dtype, ld, bias, state, q_start, q_len, state slots, requests, channels, taps, stream
+        "gb_qk_conv_state": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+        # att, lda, hd, gate, ldg, one gate a head, dtype, out, ldo, n, H, dv, stream
+        "gb_gate_rows": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _i, _i, _i, _i, _vp],
+    },
     "moe": {        # z, ldz, n, experts, correction, top, scale, shared, combine, ids, weights, stream
         "gb_moe_route": [_vp, _i, _i, _i, _vp, _i, _f, _i, _vp, _vp, _vp, _vp],
+        # z, ldz, n, experts, correction, top, scale, shared (0, 1 gate, 2 whole), softmax, renorm, groups, kept groups,
+        # combine, ids, weights, stream
+        "gb_moe_route_by": [_vp, _i, _i, _i, _vp, _i, _f, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp],
+        # z, its dtype, ld, combine, its columns, act, its dtype, lda, n, inter, experts, ff, stream
+        "gb_moe_relu2_units": [_vp, _i, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
         # gate_up, its dtype, ld, combine, its columns, act, its dtype, n, inter, experts, ff, stream
         "gb_moe_gated_units": [_vp, _i, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
         # ids, n, top, experts, rows a tile, tiles, counts, rows, pos, map, stream
@@ -150,8 +169,9 @@ _SIGS = {
         # q, q_stride, out, out_stride, dtype, positions, tok_seq, tables, table_stride, k, v, n, nh, nkv, hd, page,
         # scale, window, workspace, workspace floats, max_context, stream
         # scale, window, kept first keys, workspace, workspace floats, max_context, grouped, stream
-        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp,
-                               C.c_longlong, _i, _i, _vp],
+        # scale, window, kept first keys, run of positions, cap, sinks, workspace, workspace floats, max_context, grouped, stream
+        "gb_attention_plain": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _i, _f, _vp,
+                               _vp, C.c_longlong, _i, _i, _vp],
         "gb_attention_plain_split_floats": [_i, _i, _i, _i, _i, _i],
     },
     "attention_bf16": {
@@ -164,6 +184,15 @@ _SIGS = {
         "gb_attention_prefill_bf16": [_vp, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
                                       _f, _i, _i, _i, _vp, C.c_longlong, _vp],
         "gb_attention_prefill_parts": [_i, _i, _i, _i, _i],
+        # q, q_stride, out, out_stride, out32, ws_acc, ws_ml, positions, tables, table_stride, k, v, n_decode, nh, nkv, hd,
+        # page, scale, window, kept first keys, run of positions, cap, sinks, chunk, max_context, stream
+        "gb_attention_decode_bf16_by": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
+                                        _i, _f, _vp, _i, _i, _vp],
+        # q, q_stride, out, out_stride, out32, q_start, q_len, pos0, seq_base, n_seqs, max_q_len, max_context, tables,
+        # table_stride, k, v, nh, nkv, hd, page, scale, window, kept first keys, run of positions, cap, sinks, first_row,
+        # n_rows, part_ws, part_floats, stream
+        "gb_attention_prefill_bf16_by": [_vp, _i, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i,
+                                         _f, _i, _i, _i, _f, _vp, _i, _i, _vp, C.c_longlong, _vp],
         # the same two with the number of kept first keys after the window
         "gb_attention_decode_bf16_keep": [_vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i,
                                           _i, _i, _vp],
@@ -1106,16 +1135,20 @@ MOE_MAX_EXPERTS = 512   # moe.hip: a lane of the routing wave holds eight expert
 MOE_MAX_TOP = 16
 
 
-def moe_route(z: torch.Tensor, n_experts: int, correction: Optional[torch.Tensor], top: int, scale: float, shared: bool,
-              combine: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
-    """From router logits ``z`` (float32 [n, experts (+ 1)]): scores sigmoid(z); the ``top`` experts with the largest
-    score + correction (of equal ones the lower index); their weights score / (sum of the chosen scores + 1e-20) * scale.
+def moe_route(z: torch.Tensor, n_experts: int, correction: Optional[torch.Tensor], top: int, scale: float, shared,
+              combine: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, softmax: bool = False, renorm: bool = True,
+              groups: int = 0, keep_groups: int = 0) -> None:
+    """From router logits ``z`` (float32 [n, experts (+ 1)]): scores sigmoid(z), or with ``softmax`` the softmax over all
+    experts; the ``top`` experts with the largest score + correction (of equal ones the lower index), with ``groups`` only
+    out of the ``keep_groups`` runs of experts / groups neighbours whose best score + correction is largest; their weights
+    score * scale, with ``renorm`` divided by (the sum of the chosen scores + 1e-20).
     ``ids`` int32 and ``weights`` float32 [n, top] receive the choice, ``combine`` float32 [n, experts (+ 1)] a row of
-    weights with zeros for the others; with ``shared``, its last column is sigmoid of z's last column."""
+    weights with zeros for the others; with ``shared`` one more column for an expert that every token uses: sigmoid of
+    z's last column (True, "gate"), or 1 ("whole")."""
     _dev(z, correction, combine, ids, weights)
     n = z.shape[0]
     cols = n_experts + (1 if shared else 0)
-    if z.dtype != torch.float32 or z.dim() != 2 or z.stride(1) != 1 or z.shape[1] < cols:
+    if z.dtype != torch.float32 or z.dim() != 2 or z.stride(1) != 1 or z.shape[1] < n_experts + (1 if shared and shared != "whole" else 0):
         raise KernelError("moe_route: z must be float32 [n, experts (+ 1)] with dense rows")
     _f32_rows(combine, (n, cols), "combine")
     _f32_rows(weights, (n, top), "weights")
@@ -1123,8 +1156,28 @@ def moe_route(z: torch.Tensor, n_experts: int, correction: Optional[torch.Tensor
     if correction is not None:
         _f32_rows(correction, (n_experts,), "correction")
     lib = _lib("moe")
+    if softmax or not renorm or groups or shared == "whole":
+        _launch(lib, lib.gb_moe_route_by, _p(z), z.stride(0), n, n_experts, _p(correction), int(top), float(scale),
+                2 if shared == "whole" else 1 if shared else 0, 1 if softmax else 0, 1 if renorm else 0, int(groups),
+                int(keep_groups), _p(combine), _p(ids), _p(weights), _stream())
+        return
     _launch(lib, lib.gb_moe_route, _p(z), z.stride(0), n, n_experts, _p(correction), int(top), float(scale),
             1 if shared else 0, _p(combine), _p(ids), _p(weights), _stream())
+
+
+def moe_relu2_units(z: torch.Tensor, combine: Optional[torch.Tensor], out: torch.Tensor, n_experts: int, ff: int) -> None:
+    """out[t, j] = relu(z[t, j])^2 * combine[t, expert of column j] for units of one up matrix: columns e * ff .. of ``z``
+    and ``out`` ([n, I]) are expert e's, those from experts * ff on the shared expert's (weight in the last column of
+    ``combine``).  Without ``combine`` every weight is 1 (rows that are one expert's own)."""
+    _dev(z, combine, out)
+    n, inter = out.shape
+    if z.shape != (n, inter) or z.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("moe_relu2_units: z and out must be [n, I] with dense rows")
+    if combine is not None and (combine.dtype != torch.float32 or not combine.is_contiguous() or combine.shape[0] != n):
+        raise KernelError("moe_relu2_units: combine must be contiguous float32 [n, experts (+ 1)]")
+    lib = _lib("moe")
+    _launch(lib, lib.gb_moe_relu2_units, _p(z), dtype_code(z), z.stride(0), _p(combine), combine.shape[1] if combine is not None else 0,
+            _p(out), dtype_code(out), out.stride(0), n, inter, n_experts, ff, _stream())
 
 
 def moe_gated_units(gate_up: torch.Tensor, combine: torch.Tensor, out: torch.Tensor, n_experts: int, ff: int) -> None:
@@ -1451,6 +1504,7 @@ def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: 
 
 
 ROPE_PRODUCT_MAX_ROWS = 64
+QK_HEADS_MAX_CHANNELS = 15872   # tanhmix.hip stages a token's query and key channels in 64 KB of LDS
 
 
 def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
@@ -1523,8 +1577,12 @@ def attention_plain_split_floats(n: int, n_heads: int, head_dim: int, page_size:
 def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
                     tables: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, n_heads: int,
                     scale: float, window: int = 0, workspace: Optional[torch.Tensor] = None, max_context: int = 0,
-                    grouped: bool = False, keep_first: int = 0) -> None:
+                    grouped: bool = False, keep_first: int = 0, chunk: int = 0, softcap: float = 0.0,
+                    sinks: Optional[torch.Tensor] = None) -> None:
     """Paged attention, one block per (token, head); q may be a view into the stacked qkv rows.
+    ``chunk`` > 0 (no window then): positions are cut into runs of ``chunk`` from 0 on and a token reads the keys of its
+    own run up to itself; ``softcap`` > 0: scores pass softcap * tanh(score / softcap); ``sinks`` float32 [heads]:
+    exp(sinks[h]) joins the softmax's denominator of head h and has no value.
     ``window`` > 0: a token at position p reads keys p - window + 1 .. p, and with ``keep_first`` also keys
     0 .. keep_first - 1 wherever the window has moved past them.
     ``workspace`` (float32, ``attention_plain_split_floats`` elements) with ``max_context`` (at least the most keys a
@@ -1551,8 +1609,16 @@ def attention_plain(q: torch.Tensor, out: torch.Tensor, positions: torch.Tensor,
     _launch(lib, lib.gb_attention_plain, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), dtype_code(q), _p(positions),
                                        _p(tok_seq), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n,
                                        n_heads, nkv, hd, page_size, float(scale), int(window), int(keep_first),
+                                       int(chunk), float(softcap), _p(_sinks(sinks, n_heads)),
                                        _p(workspace), workspace.numel() if workspace is not None else 0, int(max_context),
                                        1 if grouped else 0, _stream())
+
+
+def _sinks(sinks: Optional[torch.Tensor], n_heads: int) -> Optional[torch.Tensor]:
+    if sinks is not None and (not sinks.is_cuda or sinks.dtype != torch.float32 or not sinks.is_contiguous()
+                              or sinks.numel() != n_heads):
+        raise KernelError(f"attention: sinks must be contiguous float32 [{n_heads}] on the GPU")
+    return sinks
 
 
 def tuned_attention_supports(k_pages: torch.Tensor, n_heads: int, window: int, keep_first: int = 0) -> bool:
@@ -1581,7 +1647,7 @@ def decode_chunk(n_decode: int, n_kv_heads: int, max_context: int) -> int:
 
 
 def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int,
-                     keep_first: int = 0) -> None:
+                     keep_first: int = 0, chunk: int = 0, softcap: float = 0.0, sinks: Optional[torch.Tensor] = None) -> None:
     """Rows 0..n_decode-1 of the step (requests with a single token), split over their context."""
     n_dec = ctx.host["n_decode"]
     k_pages, v_pages = cache.k_pages, cache.v_pages
@@ -1591,11 +1657,18 @@ def attention_decode(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: in
         raise KernelError("attention_decode: q must be bfloat16 [n, heads * head size], out bfloat16 or float32")
     tables = ctx.tables[cache.group]
     max_context = int(ctx.host["max_context"])
+    mask_chunk = int(chunk)   # the runs of positions a token sees; ``chunk`` below is the keys a workgroup takes
     chunk = decode_chunk(n_dec, nkv, max_context)
     splits = -(-max_context // chunk)
     ws_acc = ctx.buffer("attn_ws_acc", (n_dec * n_heads * splits * hd,), torch.float32)
     ws_ml = ctx.buffer("attn_ws_ml", (n_dec * n_heads * splits * 2,), torch.float32)
     lib = _lib("attention_bf16")
+    if mask_chunk or softcap or sinks is not None:
+        _launch(lib, lib.gb_attention_decode_bf16_by, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"),
+                1 if out.dtype == torch.float32 else 0, _p(ws_acc), _p(ws_ml), _p(ctx.positions), _p(tables), tables.stride(0),
+                _p(k_pages), _p(v_pages), n_dec, n_heads, nkv, hd, page, float(scale), int(window), int(keep_first), mask_chunk,
+                float(softcap), _p(_sinks(sinks, n_heads)), chunk, max_context, _stream())
+        return
     if keep_first or out.dtype == torch.float32:
         _launch(lib, lib.gb_attention_decode_bf16_out32 if out.dtype == torch.float32 else lib.gb_attention_decode_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ws_acc), _p(ws_ml),
                 _p(ctx.positions), _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_dec, n_heads, nkv, hd, page,
@@ -1613,7 +1686,7 @@ def _prefill_parts(max_q: int, max_ctx: int, n_heads: int, n_seqs: int, hd: int)
 
 
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: int, scale: float, window: int,
-                      keep_first: int = 0) -> None:
+                      keep_first: int = 0, chunk: int = 0, softcap: float = 0.0, sinks: Optional[torch.Tensor] = None) -> None:
     """The requests of the step that bring more than one token (they follow the single-token ones)."""
     n_dec, S = ctx.host["n_decode"], ctx.num_seqs
     k_pages, v_pages = cache.k_pages, cache.v_pages
@@ -1629,6 +1702,13 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, ctx, cache, n_heads: i
     first_row, n_rows = n_dec, q.shape[0] - n_dec
     parts = _prefill_parts(max_q, max_ctx, n_heads, S - n_dec, hd)
     ws = ctx.buffer("attn_parts", (parts * n_rows * n_heads * (hd + 2),), torch.float32) if parts > 1 else None
+    if chunk or softcap or sinks is not None:
+        _launch(lib, lib.gb_attention_prefill_bf16_by, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"),
+                1 if out.dtype == torch.float32 else 0, _p(ctx.q_start), _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q,
+                max_ctx, _p(tables), tables.stride(0), _p(k_pages), _p(v_pages), n_heads, nkv, hd, page, float(scale),
+                int(window), int(keep_first), int(chunk), float(softcap), _p(_sinks(sinks, n_heads)), first_row, n_rows, _p(ws),
+                ws.numel() if ws is not None else 0, _stream())
+        return
     if keep_first or out.dtype == torch.float32:
         _launch(lib, lib.gb_attention_prefill_bf16_out32 if out.dtype == torch.float32 else lib.gb_attention_prefill_bf16_keep, _p(q), _rows(q, "q"), _p(out), _rows(out, "out"), _p(ctx.q_start),
                 _p(ctx.q_len), _p(ctx.pos0), n_dec, S - n_dec, max_q, max_ctx, _p(tables), tables.stride(0), _p(k_pages),
@@ -1685,3 +1765,113 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
     lib = _lib("sampling")
     _launch(lib, lib.gb_sample, _p(logits), rows, vocab, _p(temperature), _p(top_k), _p(top_p), _p(min_p), _p(uniform),
                               _p(out_token), _p(out_candidates), _stream())
+
+
+# ------------------------------------------------------------------------ bounded norms, prepared heads, gates
+def _vec32(t: Optional[torch.Tensor], n: int, what: str) -> None:
+    if t is not None and (not t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n):
+        raise KernelError(f"{what} must be contiguous float32 [{n}] on the GPU")
+
+
+def tanh_norm(x: torch.Tensor, alpha: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, out: torch.Tensor,
+              rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = tanh(alpha * x[rows[r] or r]) * weight + bias; x float32 [n, d], ``alpha`` one number on the device;
+    ``out`` may be x itself."""
+    _dev(x, out, rows)
+    m, d = out.shape
+    if x.dtype != torch.float32 or x.dim() != 2 or x.shape[1] != d or (rows is None and x.shape[0] < m):
+        raise KernelError("tanh_norm: x must be float32 [n, d] with a row for every row of out")
+    _vec32(alpha, 1, "tanh_norm: alpha")
+    _vec32(weight, d, "tanh_norm: weight")
+    _vec32(bias, d, "tanh_norm: bias")
+    _i32(rows, "rows", m)
+    lib = _lib("tanhmix")
+    _launch(lib, lib.gb_tanh_norm, _p(x), _rows(x, "x"), _p(rows), _p(alpha), _p(weight), _p(bias), _p(out), dtype_code(out),
+            _rows(out, "out"), m, d, _stream())
+
+
+def tanh_norm_add(x: torch.Tensor, y: torch.Tensor, norm: tuple, slices: int = 1, then: Optional[tuple] = None,
+                  h: Optional[torch.Tensor] = None) -> None:
+    """x += tanh(alpha * y) * weight + bias with ``norm = (alpha, weight, bias)``; x float32 [n, d]; y float32 [n, d] or, with
+    ``slices`` > 1, that many such pieces one behind the other, added up in their order first.  ``then = (alpha, weight,
+    bias)`` with ``h`` [n, d]: h = tanh(alpha * x) * weight + bias of the new x, in h's type, in the same pass."""
+    _dev(x, y, h)
+    n, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or y.dtype != torch.float32 or not y.is_contiguous() \
+            or y.numel() < slices * n * d:
+        raise KernelError("tanh_norm_add: x and y must be contiguous float32, y with a piece of x's size for every slice")
+    for a, w, b in (norm,) + ((then,) if then is not None else ()):
+        _vec32(a, 1, "tanh_norm_add: alpha")
+        _vec32(w, d, "tanh_norm_add: weight")
+        _vec32(b, d, "tanh_norm_add: bias")
+    if (then is None) != (h is None) or (h is not None and (tuple(h.shape) != (n, d) or not h.is_contiguous())):
+        raise KernelError("tanh_norm_add: the next norm and the rows it writes come together, rows contiguous [n, d]")
+    a2, w2, b2 = then if then is not None else (None, None, None)
+    lib = _lib("tanhmix")
+    _launch(lib, lib.gb_tanh_norm_add, _p(x), _p(y), int(slices), n * d, _p(norm[0]), _p(norm[1]), _p(norm[2]), _p(a2), _p(w2),
+            _p(b2), _p(h), dtype_code(h) if h is not None else F32, n, d, _stream())
+
+
+def qk_heads(proj: torch.Tensor, ctx, out: torch.Tensor, head_cols: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int,
+             eps: float, joint: bool, norm_q: Optional[torch.Tensor], norm_k: Optional[torch.Tensor],
+             bias: Optional[torch.Tensor] = None, wconv: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
+             cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot: int = 0, magnitude: float = 1.0,
+             neighbours: bool = True, tied: bool = False, slots: Optional[torch.Tensor] = None,
+             k_pages: Optional[torch.Tensor] = None, v_pages: Optional[torch.Tensor] = None) -> None:
+    """The query, key and value heads of every row of the step as attention reads them, ``out`` [n, (heads + 2 kv heads) *
+    head_cols], from the stacked projections ``proj`` ([n, query channels | key channels | value channels | ...]; with
+    ``tied`` there are no value channels: the key channels, biased and convolved, are the values):
+    ``bias`` (float32, one a channel) is added; ``wconv`` ([query + key channels, taps] float32) convolves every query and
+    key channel over the request's earlier rows and its ``state`` slot ([slots, taps - 1, channels] float32, moved on here
+    in a step of single tokens, else by ``qk_conv_state``); an RMS norm over all query (key) channels at once with a weight a
+    channel (``joint``) or over each head with ``dim`` weights that the heads share; the first ``rot`` channels of each
+    head turned by the rows' angles (``cos``, ``sin`` float32 [n, rot / 2], times ``magnitude``), channel 2i with 2i + 1
+    (``neighbours``) or i with i + rot / 2.  With ``slots`` keys and values also go to their pages."""
+    _dev(proj, out, bias, wconv, state, cos, sin, slots, k_pages, v_pages, norm_q, norm_k)
+    n = proj.shape[0]
+    channels = (n_heads + n_kv_heads) * dim
+    taps = 0
+    if wconv is not None:
+        taps = wconv.shape[1]
+        _f32_rows(wconv, (channels, taps), "qk_heads: wconv")
+        if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
+                         or tuple(state.shape[1:]) != (taps - 1, channels)):
+            raise KernelError(f"qk_heads: state must be contiguous float32 [slots, {taps - 1}, {channels}]")
+    if proj.dtype != out.dtype or out.shape[0] != n or out.shape[1] != (n_heads + 2 * n_kv_heads) * head_cols:
+        raise KernelError("qk_heads: out must be [n, (heads + 2 kv heads) * head_cols] of the projections' type")
+    _vec32(bias, channels + (0 if tied else n_kv_heads * vdim), "qk_heads: bias")
+    for w, size, what in ((norm_q, n_heads * dim if joint else dim, "norm_q"), (norm_k, n_kv_heads * dim if joint else dim, "norm_k")):
+        _vec32(w, size, f"qk_heads: {what}")
+    if rot:
+        _f32_rows(cos, (n, rot // 2), "qk_heads: cos")
+        _f32_rows(sin, (n, rot // 2), "qk_heads: sin")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots", n)
+        _, nkv, page, hd = _check_pages(k_pages, v_pages, proj.dtype, "qk_heads")
+        if nkv != n_kv_heads or hd != head_cols:
+            raise KernelError("qk_heads: the pages hold other heads than these")
+    single = 1 if ctx.host["n_decode"] == ctx.num_seqs else 0
+    lib = _lib("tanhmix")
+    _launch(lib, lib.gb_qk_heads, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(bias), _p(wconv), int(taps), _p(state),
+            _p(ctx.tok_seq), _p(ctx.q_start), _p(ctx.pos0), _p(ctx.state_slots), single, _p(norm_q), _p(norm_k), float(eps),
+            1 if joint else 0, _p(cos), _p(sin), int(rot), float(magnitude), 1 if neighbours else 0, 1 if tied else 0, _p(out),
+            _rows(out, "out"), int(head_cols), _p(slots), _p(k_pages), _p(v_pages), int(page), n, n_heads, n_kv_heads, dim, vdim,
+            _stream())
+    if taps > 1 and not single:
+        _launch(lib, lib.gb_qk_conv_state, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(bias), _p(state), _p(ctx.q_start),
+                _p(ctx.q_len), _p(ctx.state_slots), ctx.num_seqs, channels, int(taps), _stream())
+
+
+def gate_rows(att: torch.Tensor, head_cols: int, gate: torch.Tensor, out: torch.Tensor, n_heads: int, vdim: int,
+              per_head: bool) -> None:
+    """out[:, h, c] = att[:, h, c] * sigmoid(g) for c < vdim, g = gate[:, h] (``per_head``) or gate[:, h, c]: ``att`` [n, heads *
+    head_cols], ``out`` [n, heads * vdim]; ``gate`` may be columns of a wider tensor."""
+    _dev(att, gate, out)
+    n = att.shape[0]
+    if att.dtype != gate.dtype or att.dtype != out.dtype or att.shape[1] != n_heads * head_cols or out.shape != (n, n_heads * vdim) \
+            or gate.shape != (n, n_heads if per_head else n_heads * vdim):
+        raise KernelError("gate_rows: att [n, heads * head_cols], gate [n, heads (* vdim)] and out [n, heads * vdim] of one type")
+    lib = _lib("tanhmix")
+    _launch(lib, lib.gb_gate_rows, _p(att), _rows(att, "att"), int(head_cols), _p(gate), _rows(gate, "gate"), 1 if per_head else 0,
+            dtype_code(att), _p(out), _rows(out, "out"), n, n_heads, vdim, _stream())

@@ -20,9 +20,13 @@ from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding,
 
 
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, n_heads: int, scale: float,
-                    window: int, keep_first: int = 0) -> None:
+                    window: int, keep_first: int = 0, chunk: int = 0, softcap: float = 0.0,
+                    sinks: Optional[torch.Tensor] = None) -> None:
     """Attention of every row of the step over its request's pages.  ``window`` > 0: a token reads the last so many
     keys up to its own, and with ``keep_first`` the request's first so many keys as well, wherever they lie.
+    ``chunk`` > 0 (instead of a window): positions are cut into runs of so many, counted from the request's first, and a
+    token reads the keys of its own run up to itself.  ``softcap`` > 0: scores pass softcap * tanh(score / softcap).
+    ``sinks`` (float32 [heads]): exp(sinks[h]) joins the softmax's denominator of head h and has no value.
 
     float32 always takes the plain kernel.  bfloat16 takes the tuned kernels where they apply: requests with
     one row go to the split-context decode kernel, longer portions to the matrix-core prefill kernel; a step
@@ -40,11 +44,11 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, 
             ws = ctx.buffer("attention_plain_parts", (floats,), torch.float32) if floats else None
             ops.attention_plain(q[a:b], out[a:b], ctx.positions[a:b], ctx.tok_seq[a:b], tables, cache.k_pages, cache.v_pages,
                                 n_heads, scale, window, workspace=ws, max_context=longest, grouped=grouped,
-                                keep_first=keep_first)
+                                keep_first=keep_first, chunk=chunk, softcap=softcap, sinks=sinks)
 
         # the rows of requests with one token come first; many rows of prompt portions go eight rows a workgroup
         n, n_decode = q.shape[0], ctx.host["n_decode"]
-        if n - n_decode >= ops.PLAIN_GROUP_MIN_ROWS and window == 0:
+        if n - n_decode >= ops.PLAIN_GROUP_MIN_ROWS and window == 0 and chunk == 0:
             if n_decode > 0:
                 rows(0, n_decode, False)
             rows(n_decode, n, True)
@@ -53,9 +57,9 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, cache: LayerCache, 
         return
     n_decode = ctx.host["n_decode"]
     if n_decode > 0:
-        ops.attention_decode(q, out, ctx, cache, n_heads, scale, window, keep_first)
+        ops.attention_decode(q, out, ctx, cache, n_heads, scale, window, keep_first, chunk, softcap, sinks)
     if n_decode < ctx.num_seqs:
-        ops.attention_prefill(q, out, ctx, cache, n_heads, scale, window, keep_first)
+        ops.attention_prefill(q, out, ctx, cache, n_heads, scale, window, keep_first, chunk, softcap, sinks)
 
 
 class PagedAttention(Mixer):
@@ -517,4 +521,143 @@ class DifferentialAttention(Mixer):
         if store:   # the caller's norm adds the slices of a product that divides k
             return product_in_slices(ctx, o, self.wo, residual)
         product(ctx, o, self.wo, residual, accumulate=True)
+        return None
+
+
+class GatedAttention(Mixer):
+    """Grouped-query attention whose heads are gated before the output projection, with a sink in the softmax, and whose
+    query and key heads are prepared in one pass.  Every option is a constructor argument:
+
+    * ``bias``: biases on the query, key and value projections (``q.b``, ``k.b``, ``v.b``);
+    * ``taps`` > 0: a short causal convolution over time on every query and key channel right after the projection
+      (``q.conv``, ``k.conv`` [channels, taps], zeros before the request's first token); the request's last taps - 1
+      projections are its state;
+    * ``tied_values``: no value projection: the key channels as they leave the convolution are the value heads;
+    * ``qk_norm``: "joint": one RMS norm over all query channels (and one over all key channels) before they are cut into
+      heads, a weight a channel (``q.norm`` [heads * dim]); "head": every head over its ``dim`` channels with ``dim``
+      weights that the heads share;
+    * the first ``rot_dims`` channels of every query and key head turn with the position: ``rot_pairs`` "neighbours"
+      (channel 2i with 2i + 1) or "halves" (i with i + rot_dims / 2), frequencies base^(-2i / rot_dims), with
+      ``rot_scaling = (factor, original, fast, slow)`` stretched as ``parts.rotary.Rotary`` says;
+    * scores q . k * ``scale``, with ``softcap`` > 0 then softcap * tanh(score / softcap); ``chunk`` > 0: a token sees the
+      keys of its own run of ``chunk`` positions (runs counted from the request's first token), else all earlier keys;
+    * ``sink``: "zero": one is added to the softmax's denominator (a sink of score 0); "learned": exp(sink_h), one number a
+      head (``sink``); None: a plain softmax;
+    * ``gate``: "head": head h times sigmoid(W_g h)_h (``g`` [heads, width]); "channel": every channel of the heads times
+      its own sigmoid (``g`` [heads * vdim, width]); the gate reads the mixer's input;
+    * the output projection ``o`` on the gated heads.
+
+    One product makes queries, keys, values and gates; ``ops.qk_heads`` prepares the heads (and writes the cache in steps
+    of few rows); the framework's paged attention kernels do the rest."""
+    replayable = True
+    accepts_store = True
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: float, eps: float,
+                 bias: bool = False, taps: int = 0, tied_values: bool = False, qk_norm: str = "head", rot_dims: int = 0,
+                 rot_base: float = 10000.0, rot_pairs: str = "halves", rot_scaling=None, softcap: float = 0.0, chunk: int = 0,
+                 sink: Optional[str] = None, gate: str = "channel"):
+        from .rotary import Rotary
+        if n_heads % n_kv_heads:
+            raise ValueError(f"{n_heads} query heads are not a multiple of {n_kv_heads} key heads")
+        if rot_dims % 2 or not 0 <= rot_dims <= dim:
+            raise ValueError(f"{rot_dims} rotated channels: an even number up to the key size {dim}")
+        if tied_values and vdim != dim:
+            raise ValueError(f"values that are the keys have the keys' size: dim {dim}, vdim {vdim}")
+        if qk_norm not in ("joint", "head") or rot_pairs not in ("neighbours", "halves") or sink not in (None, "zero", "learned") \
+                or gate not in ("head", "channel"):
+            raise ValueError("qk_norm: joint | head; rot_pairs: neighbours | halves; sink: None | zero | learned; gate: head | channel")
+        self.width, self.n_heads, self.n_kv_heads, self.dim, self.vdim = width, n_heads, n_kv_heads, dim, vdim
+        self.scale, self.eps, self.bias, self.taps, self.tied_values = float(scale), float(eps), bool(bias), int(taps), bool(tied_values)
+        self.qk_norm, self.rot_dims, self.rot_pairs, self.softcap, self.chunk = qk_norm, int(rot_dims), rot_pairs, float(softcap), int(chunk)
+        self.sink, self.gate = sink, gate
+        self.head_cols = cache_head_cols(dim, vdim)
+        self.channels = (n_heads + n_kv_heads) * dim
+        self.value_cols = 0 if tied_values else n_kv_heads * vdim
+        self.gate_cols = n_heads if gate == "head" else n_heads * vdim
+        self.position = Rotary(rot_dims, rot_base, rot_scaling) if rot_dims else None
+        self.cache_spec = CacheSpec(n_kv_heads, self.head_cols, FULL, 0)
+        self.state_spec = StateSpec((self.taps - 1, self.channels), torch.float32, 0.0) if self.taps > 1 else None
+        self.w_in = self.wo = self.b_in = self.wconv = self.norm_q = self.norm_k = self.sinks = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        H, G, D, V = self.n_heads, self.n_kv_heads, self.dim, self.vdim
+        specs = {"q": TensorSpec((H * D, self.width)), "k": TensorSpec((G * D, self.width))}
+        if not self.tied_values:
+            specs["v"] = TensorSpec((G * V, self.width))
+        if self.bias:
+            specs["q.b"] = TensorSpec((H * D,), kind="f32")
+            specs["k.b"] = TensorSpec((G * D,), kind="f32")
+            if not self.tied_values:
+                specs["v.b"] = TensorSpec((G * V,), kind="f32")
+        joint = self.qk_norm == "joint"
+        specs["q.norm"] = TensorSpec((H * D if joint else D,), kind="f32", init="ones")
+        specs["k.norm"] = TensorSpec((G * D if joint else D,), kind="f32", init="ones")
+        if self.taps:
+            specs["q.conv"] = TensorSpec((H * D, self.taps), kind="f32")
+            specs["k.conv"] = TensorSpec((G * D, self.taps), kind="f32")
+        if self.sink == "learned":
+            specs["sink"] = TensorSpec((H,), kind="f32")
+        specs["g"] = TensorSpec((self.gate_cols, self.width))
+        specs["o"] = TensorSpec((self.width, H * V))
+        return specs
+
+    def load(self, tensors):
+        parts = [tensors["q"], tensors["k"]] + ([] if self.tied_values else [tensors["v"]]) + [tensors["g"]]
+        self.w_in = _stack_rows(parts, self.width)   # one product reads the mixer's input for all of them
+        self.wo = tensors["o"].contiguous()
+        if self.bias:
+            self.b_in = torch.cat([tensors["q.b"], tensors["k.b"]] + ([] if self.tied_values else [tensors["v.b"]])).float().contiguous()
+        self.norm_q, self.norm_k = tensors["q.norm"].float().contiguous(), tensors["k.norm"].float().contiguous()
+        if self.taps:
+            self.wconv = torch.cat([tensors["q.conv"], tensors["k.conv"]], 0).float().contiguous()
+        if self.sink == "learned":
+            self.sinks = tensors["sink"].float().contiguous()
+        elif self.sink == "zero":
+            self.sinks = torch.zeros(self.n_heads, dtype=torch.float32, device=self.wo.device)
+
+    def streamed_matrices(self):
+        return [self.w_in, self.wo]
+
+    def problems(self, dtype, page_size):
+        out = []
+        if self.head_cols > ops.MAX_HEAD_DIM:
+            out.append(("dim", f"heads of {max(self.dim, self.vdim)} channels are above {ops.MAX_HEAD_DIM}, the largest head "
+                               f"the attention kernels take"))
+        if self.taps > ops.CONV_MAX_TAPS:
+            out.append(("taps", f"{self.taps} is above {ops.CONV_MAX_TAPS}, the longest convolution the kernel takes"))
+        if self.channels > ops.QK_HEADS_MAX_CHANNELS:
+            out.append(("dim", f"{self.channels} query and key channels a token are above {ops.QK_HEADS_MAX_CHANNELS}, the most "
+                               f"the kernel that prepares the heads stages"))
+        return out
+
+    def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):
+        """Adds the mixed rows into ``residual``; with ``store`` writes them there instead (float32 either way) or leaves
+        them in slices, and returns what ``product_in_slices`` does."""
+        if cache is None or cache.k_pages is None or (self.taps > 1 and cache.state is None):
+            raise ValueError("GatedAttention needs a layer cache with pages (and state, with a convolution)")
+        n = h.shape[0]
+        H, G, V, hc = self.n_heads, self.n_kv_heads, self.vdim, self.head_cols
+        proj = ctx.buffer("gated_proj", (n, self.w_in.shape[0]), ctx.dtype)   # [q | k | v | gate]
+        product(ctx, h, self.w_in, proj)
+        cos, sin = self.position.table(ctx) if self.position is not None else (None, None)
+        heads = ctx.buffer("gated_heads", (n, (H + 2 * G) * hc), ctx.dtype)
+        slots = ctx.slots[cache.group] if cache.writable else None
+        direct = slots is not None and n <= ops.ROPE_PRODUCT_MAX_ROWS
+        ops.qk_heads(proj, ctx, heads, hc, H, G, self.dim, V, self.eps, self.qk_norm == "joint", self.norm_q, self.norm_k,
+                     bias=self.b_in, wconv=self.wconv, state=cache.state if self.taps > 1 else None, cos=cos, sin=sin,
+                     rot=self.rot_dims, magnitude=self.position.magnitude if self.position is not None else 1.0,
+                     neighbours=self.rot_pairs == "neighbours", tied=self.tied_values, slots=slots if direct else None,
+                     k_pages=cache.k_pages, v_pages=cache.v_pages)
+        if slots is not None and not direct:
+            # many rows: the kernel that takes a step's keys and values to their pages in whole lines
+            ops.rope_store(heads, None, None, slots, cache.k_pages, cache.v_pages, H, G, hc, rotate=False,
+                           portions=ctx.portions())
+        att = ctx.buffer("att", (n, H * hc), ctx.dtype)
+        paged_attention(ctx, heads[:, :H * hc], att, cache, H, self.scale, 0, 0, self.chunk, self.softcap, self.sinks)
+        gated = ctx.buffer("gated_rows", (n, H * V), ctx.dtype)
+        at = self.channels + self.value_cols
+        ops.gate_rows(att, hc, proj[:, at:at + self.gate_cols], gated, H, V, self.gate == "head")
+        if store:   # the caller's pass over the rows adds the slices of a product that divides k
+            return product_in_slices(ctx, gated, self.wo, residual)
+        product(ctx, gated, self.wo, residual, accumulate=True)
         return None

@@ -192,3 +192,56 @@ class OutputNormBlock(Block):
         made, slices = self.ffn.forward(ctx, rows, y, store=True) or (y, 1)
         self.ffn_norm.add_normed(ctx, made, x, rounded=handed, slices=slices, conv=emit)
         return handed
+
+
+class SandwichBlock(Block):
+    """Every sublayer between two norms: x += norm1b(mixer(norm1(x))), then x += norm2b(feed-forward(norm2(x))); the
+    feed-forward (with its two norms) may be absent.  The sublayers write their rows into a 32-bit buffer
+    (``accepts_store``) or leave them in the slices of a product that divides k, and the pass of the norm behind a
+    sublayer is the pass that adds into the residual.  The norms are ``TanhNorm``s (or anything with ``add_normed(ctx, y,
+    x, slices=, then=, rounded=)``): a norm that needs no statistic of the row can also be applied to the new residual in
+    that same pass, so the rows the feed-forward reads, and the rows the next block's mixer reads, come out of the pass
+    before them."""
+    replayable = True
+
+    def __init__(self, norm1, mixer: Mixer, norm1b, norm2=None, ffn: Optional[FeedForward] = None, norm2b=None,
+                 names=("norm1", "mix", "norm1b", "norm2", "mlp", "norm2b")):
+        for part in (mixer, ffn):
+            if part is not None and not getattr(part, "accepts_store", False):
+                raise ValueError(f"{type(part).__name__} cannot write its rows instead of adding them (accepts_store)")
+        if not ((ffn is None) == (norm2 is None) == (norm2b is None)):
+            raise ValueError("a feed-forward and its two norms come together")
+        self.norm1, self.mixer, self.norm1b, self.norm2, self.ffn, self.norm2b = norm1, mixer, norm1b, norm2, ffn, norm2b
+        self.names = tuple(names)
+
+    def children(self) -> Dict[str, Part]:
+        parts = (self.norm1, self.mixer, self.norm1b, self.norm2, self.ffn, self.norm2b)
+        return {name: part for name, part in zip(self.names, parts) if part is not None}
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return self.mixer.cache_spec
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return self.mixer.state_spec
+
+    def entry_rows(self, ctx, n: int, cache: Optional[LayerCache]):
+        """The norm this block begins with, if the pass that makes the residual before it may also make the rows this
+        block's mixer reads (``forward(..., pre=)`` then takes them); else None."""
+        return self.norm1 if hasattr(self.norm1, "spec") else None
+
+    def forward(self, ctx, x, cache: Optional[LayerCache], pre=None, emit=None):
+        """``pre``: the rows this block's mixer reads, made by the block before; ``emit``: the ``entry_rows`` of the block
+        after.  Returns the rows for that block if the last norm's pass made them."""
+        n, width = x.shape
+        h = pre if pre is not None else self.norm1.forward(ctx, x)
+        y = ctx.buffer("sublayer_y", (n, width), torch.float32)
+        made, slices = self.mixer.forward(ctx, h, y, cache, store=True) or (y, 1)
+        handed = ctx.buffer("h_handed", (n, width), ctx.dtype) if emit is not None else None
+        if self.ffn is None:
+            self.norm1b.add_normed(ctx, made, x, slices=slices, then=emit, rounded=handed)
+            return handed
+        rows = ctx.buffer("h", (n, width), ctx.dtype)
+        self.norm1b.add_normed(ctx, made, x, slices=slices, then=self.norm2, rounded=rows)
+        made, slices = self.ffn.forward(ctx, rows, y, store=True) or (y, 1)
+        self.norm2b.add_normed(ctx, made, x, slices=slices, then=emit, rounded=handed)
+        return handed

@@ -14,12 +14,17 @@ from .base import LayerCache, Part, StateSpec, TensorSpec, needs_multiple_of_8, 
 class Embedding(Part):
     replayable = True
 
-    def __init__(self, vocab: int, width: int, scale: float = 1.0):
+    def __init__(self, vocab: int, width: int, scale: float = 1.0, norm: Optional[Part] = None):
         self.vocab, self.width, self.scale = vocab, width, float(scale)
+        #: a norm of the embedded rows, applied in place to the 32-bit rows (anything with ``in_place(ctx, x)``)
+        self.norm = norm
         self.table: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {"weight": TensorSpec((self.vocab, self.width))}
+
+    def children(self) -> Dict[str, Part]:
+        return {"norm": self.norm} if self.norm is not None else {}
 
     def load(self, tensors):
         self.table = tensors["weight"].contiguous()
@@ -27,6 +32,10 @@ class Embedding(Part):
     def forward(self, ctx, out):
         """``out`` [n, width], or [streams, n, width]: every stream starts as the embedding."""
         ops.embed(self.table, ctx.token_ids, out, self.scale)
+        if self.norm is not None:
+            if out.dim() != 2:
+                raise ValueError("a normed embedding fills one residual, not several streams")
+            self.norm.in_place(ctx, out)
 
 
 class PairHashEmbedding(Embedding):

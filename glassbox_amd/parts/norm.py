@@ -1,7 +1,8 @@
 """RMS norm: out = g * (x / sqrt(mean(x^2) + eps)), sums in 32-bit
 (crates/glassbox-core/src/model.rs:94-100).  With ``offset`` the checkpoint holds the weight minus ``offset`` and
 g = offset + w, added in 32-bit when the weights are loaded and kept in 32-bit.  ``ScalarRMSNorm`` has one number for all
-coordinates and can also norm a sublayer's *output* on its way into the residual."""
+coordinates and can also norm a sublayer's *output* on its way into the residual.  ``TanhNorm`` computes no statistic
+of the row at all: out = tanh(alpha x) * w + b with one number alpha."""
 from __future__ import annotations
 
 from typing import Dict, Optional, Tuple
@@ -82,3 +83,47 @@ class ScalarRMSNorm(Norm):
         """x += g * y / sqrt(mean(y^2) + eps) (both float32; ``slices`` > 1: y is the sum of that many pieces);
         ``rounded`` receives the new x in its own type, or with ``conv=(weight, state)`` what a ``TimeConv`` makes of it."""
         ops.norm_add(x, y, self.gain, self.eps, rounded, slices=slices, conv=conv, ctx=ctx)
+
+
+class TanhNorm(Norm):
+    """out = tanh(alpha * x) * weight + bias: ``alpha`` a single number (a tensor without dimensions), weight and bias a
+    number a coordinate; no mean, no variance.  As a norm of rows (``forward``) it writes the rows a sublayer reads;
+    ``add_normed`` norms a sublayer's output y on its way into the residual, and since nothing of a row has to be
+    summed first, the same pass can also write the rows that the next norm of this kind makes of the new residual
+    (``then=``).  32-bit arithmetic in both precisions."""
+    replayable = True
+    taped = True
+
+    def __init__(self, width: int):
+        self.width = width
+        self.alpha: Optional[torch.Tensor] = None     # [1]
+        self.weight: Optional[torch.Tensor] = None    # [width]
+        self.bias: Optional[torch.Tensor] = None      # [width]
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {"weight": TensorSpec((self.width,), kind="f32", init="ones"),
+                "bias": TensorSpec((self.width,), kind="f32", init="normal"),
+                "alpha": TensorSpec((), kind="f32", init="ones")}
+
+    def load(self, tensors):
+        self.alpha = tensors["alpha"].float().reshape(1).contiguous()
+        self.weight = tensors["weight"].float().contiguous()
+        self.bias = tensors["bias"].float().contiguous()
+
+    def spec(self) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        return (self.alpha, self.weight, self.bias)
+
+    def forward(self, ctx, x, rows=None, out_name="h"):
+        m = x.shape[0] if rows is None else rows.numel()
+        out = ctx.buffer(out_name, (m, self.width), ctx.dtype)
+        ops.tanh_norm(x, self.alpha, self.weight, self.bias, out, rows)
+        return out
+
+    def in_place(self, ctx, x) -> None:
+        """x = norm(x) on float32 rows (an embedding's output)."""
+        ops.tanh_norm(x, self.alpha, self.weight, self.bias, x)
+
+    def add_normed(self, ctx, y, x, slices: int = 1, then: Optional["TanhNorm"] = None, rounded=None) -> None:
+        """x += norm(y) (both float32; ``slices`` > 1: y is the sum of that many pieces); with ``then`` and ``rounded``:
+        rounded = then(new x)."""
+        ops.tanh_norm_add(x, y, self.spec(), slices=slices, then=then.spec() if then is not None else None, h=rounded)

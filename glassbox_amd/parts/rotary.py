@@ -6,8 +6,15 @@ computed on the host exactly as the reference does (64-bit power, rounded to
 32-bit); the angle is a 32-bit product and its sine and cosine are evaluated
 in 64-bit on the device, once per step for all layers that share the
 encoding's constants.
+
+``scaling = (factor, original, fast, slow)`` stretches the slow turns for contexts beyond ``original`` positions:
+with index(t) = R ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(index(fast)), 0), hi = min(ceil(index(slow)),
+R - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency of pair i is f_i / factor * ramp_i +
+f_i * (1 - ramp_i); ``magnitude`` = 0.1 ln(factor) + 1 is what the caller multiplies cosine and sine by.
 """
 from __future__ import annotations
+
+import math
 
 import numpy as np
 import torch
@@ -20,26 +27,43 @@ class Rotary(PositionEncoding):
     replayable = True
     taped = True
 
-    def __init__(self, head_dim: int, theta: float):
+    def __init__(self, head_dim: int, theta: float, scaling=None):
         if head_dim % 2:
             raise ValueError(f"rotary pairs need an even head size, got {head_dim}")
         self.head_dim = head_dim
         self.theta = float(np.float32(theta))  # the reference holds theta in 32-bit (model.rs:18)
         half = head_dim // 2
-        self.inv_host = np.array([np.float32(1.0 / (self.theta ** ((2 * i) / head_dim))) for i in range(half)],
-                                 dtype=np.float32)
+        self.scaling = None if scaling is None else tuple(float(v) for v in scaling)
+        self.magnitude = 1.0
+        if self.scaling is None:
+            self.inv_host = np.array([np.float32(1.0 / (self.theta ** ((2 * i) / head_dim))) for i in range(half)],
+                                     dtype=np.float32)
+        else:
+            factor, original, fast, slow = self.scaling
+            if not (factor > 0 and original > 0 and fast > 0 and slow > 0 and self.theta > 1):
+                raise ValueError(f"rotary scaling (factor, original, fast, slow) = {self.scaling}: all must be positive")
+            index = lambda turns: head_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+            lo, hi = max(math.floor(index(fast)), 0), min(math.ceil(index(slow)), head_dim - 1)
+            inv = []
+            for i in range(half):
+                f = 1.0 / (self.theta ** ((2 * i) / head_dim))
+                ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+                inv.append(np.float32(f / factor * ramp + f * (1.0 - ramp)))
+            self.inv_host = np.array(inv, dtype=np.float32)
+            self.magnitude = 0.1 * math.log(factor) + 1.0
         self._inv_dev = None
 
     def table(self, ctx):
         """cos and sin [tokens, hd/2] for this step's positions, shared by every layer with the same constants."""
-        key = ("rotary", self.head_dim, self.theta)
+        key = ("rotary", self.head_dim, self.theta, self.scaling)
         hit = ctx.memo.get(key)
         if hit is None:
             if self._inv_dev is None or self._inv_dev.device != ctx.device:
                 self._inv_dev = torch.from_numpy(self.inv_host).to(ctx.device)
             half = self.head_dim // 2
-            cos = ctx.buffer(f"rope_cos_{self.head_dim}_{self.theta}", (ctx.n, half), torch.float32)
-            sin = ctx.buffer(f"rope_sin_{self.head_dim}_{self.theta}", (ctx.n, half), torch.float32)
+            tag = f"{self.head_dim}_{self.theta}" + ("" if self.scaling is None else "_" + "_".join(map(str, self.scaling)))
+            cos = ctx.buffer(f"rope_cos_{tag}", (ctx.n, half), torch.float32)
+            sin = ctx.buffer(f"rope_sin_{tag}", (ctx.n, half), torch.float32)
             ops.rope_table(ctx.positions, self._inv_dev, cos, sin)
             hit = (cos, sin)
             ctx.memo[key] = hit
@@ -54,7 +78,7 @@ class Rotary(PositionEncoding):
 
 
     def fuse_spec(self, ctx, head_dim: int):
-        return self.table(ctx) if head_dim == self.head_dim else None
+        return self.table(ctx) if head_dim == self.head_dim and self.magnitude == 1.0 else None
 
 
 class NoPosition(PositionEncoding):
