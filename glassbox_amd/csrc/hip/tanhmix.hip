@@ -261,12 +261,14 @@ extern "C" int gb_tanh_norm_add(float* x, const float* y, int slices, long long 
   return launched("tanh_norm_add");
 }
 
+// flags: 1 = every request brings one row (the slots are moved on here), 2 = one norm over all query (key) channels,
+// 4 = neighbouring channels pair up, 8 = the values are the keys.
 extern "C" int gb_qk_heads(const void* proj, int dtype, int ld, const float* bias, const float* wconv, int taps, float* state,
                            const int32_t* tok_seq, const int32_t* q_start, const int32_t* pos0, const int32_t* state_slots,
-                           int single, const float* wq, const float* wk, float eps, int joint, const float* cosv,
-                           const float* sinv, int rot, float mag, int neighbours, int tied, void* out, int ldo, int hd,
-                           const int32_t* slots, void* k_pages, void* v_pages, int page_size, int n, int nh, int nkv, int dk,
-                           int dv, hipStream_t stream) {
+                           int flags, const float* wq, const float* wk, float eps, const float* cosv, const float* sinv, int rot,
+                           float mag, void* out, int ldo, int hd, const int32_t* slots, void* k_pages, void* v_pages,
+                           int page_size, int n, int nh, int nkv, int dk, int dv, hipStream_t stream) {
+  const int single = flags & 1, joint = (flags >> 1) & 1, neighbours = (flags >> 2) & 1, tied = (flags >> 3) & 1;
   GB_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0 && hd >= dk && hd >= dv, "qk_heads: bad sizes nh=%d nkv=%d dk=%d dv=%d hd=%d", nh, nkv, dk, dv, hd);
   GB_REQUIRE(!tied || dv == dk, "qk_heads: values that are the keys have the keys' size (dk=%d, dv=%d)", dk, dv);
   const int channels = (nh + nkv) * dk;

@@ -94,9 +94,9 @@ _SIGS = {
         "gb_tanh_norm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
         # x, y, slices, slice stride, alpha, w, b, next alpha, w, b, h, its dtype, n, d, stream
         "gb_tanh_norm_add": [_vp, _vp, _i, C.c_longlong, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
-        # proj, dtype, ld, bias, wconv, taps, state, tok_seq, q_start, pos0, state slots, single, wq, wk, eps, joint, cos, sin,
-        # rot, mag, neighbours, tied, out, ldo, hd, slots, k, v, page, n, H, G, dk, dv, stream
-        "gb_qk_heads": [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _f, _i, _vp, _vp, _i, _f, _i, _i, _vp, _i,
+        # proj, dtype, ld, bias, wconv, taps, state, tok_seq, q_start, pos0, state slots, flags, wq, wk, eps, cos, sin,
+        # rot, mag, out, ldo, hd, slots, k, v, page, n, H, G, dk, dv, stream
+        "gb_qk_heads": [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _f, _vp, _i,
                         _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
         # proj, dtype, ld, bias, state, q_start, q_len, state slots, requests, channels, taps, stream
         "gb_qk_conv_state": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
@@ -1854,10 +1854,10 @@ def qk_heads(proj: torch.Tensor, ctx, out: torch.Tensor, head_cols: int, n_heads
     single = 1 if ctx.host["n_decode"] == ctx.num_seqs else 0
     lib = _lib("tanhmix")
     _launch(lib, lib.gb_qk_heads, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(bias), _p(wconv), int(taps), _p(state),
-            _p(ctx.tok_seq), _p(ctx.q_start), _p(ctx.pos0), _p(ctx.state_slots), single, _p(norm_q), _p(norm_k), float(eps),
-            1 if joint else 0, _p(cos), _p(sin), int(rot), float(magnitude), 1 if neighbours else 0, 1 if tied else 0, _p(out),
-            _rows(out, "out"), int(head_cols), _p(slots), _p(k_pages), _p(v_pages), int(page), n, n_heads, n_kv_heads, dim, vdim,
-            _stream())
+            _p(ctx.tok_seq), _p(ctx.q_start), _p(ctx.pos0), _p(ctx.state_slots),
+            single | (2 if joint else 0) | (4 if neighbours else 0) | (8 if tied else 0), _p(norm_q), _p(norm_k), float(eps),
+            _p(cos), _p(sin), int(rot), float(magnitude), _p(out), _rows(out, "out"), int(head_cols), _p(slots), _p(k_pages),
+            _p(v_pages), int(page), n, n_heads, n_kv_heads, dim, vdim, _stream())
     if taps > 1 and not single:
         _launch(lib, lib.gb_qk_conv_state, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(bias), _p(state), _p(ctx.q_start),
                 _p(ctx.q_len), _p(ctx.state_slots), ctx.num_seqs, channels, int(taps), _stream())

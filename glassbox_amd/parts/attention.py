@@ -550,6 +550,7 @@ class GatedAttention(Mixer):
     One product makes queries, keys, values and gates; ``ops.qk_heads`` prepares the heads (and writes the cache in steps
     of few rows); the framework's paged attention kernels do the rest."""
     replayable = True
+    taped = True
     accepts_store = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: float, eps: float,

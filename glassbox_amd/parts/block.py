@@ -203,6 +203,7 @@ class SandwichBlock(Block):
     that same pass, so the rows the feed-forward reads, and the rows the next block's mixer reads, come out of the pass
     before them."""
     replayable = True
+    taped = True
 
     def __init__(self, norm1, mixer: Mixer, norm1b, norm2=None, ffn: Optional[FeedForward] = None, norm2b=None,
                  names=("norm1", "mix", "norm1b", "norm2", "mlp", "norm2b")):
@@ -225,9 +226,9 @@ class SandwichBlock(Block):
         return self.mixer.state_spec
 
     def entry_rows(self, ctx, n: int, cache: Optional[LayerCache]):
-        """The norm this block begins with, if the pass that makes the residual before it may also make the rows this
-        block's mixer reads (``forward(..., pre=)`` then takes them); else None."""
-        return self.norm1 if hasattr(self.norm1, "spec") else None
+        """``(alpha, weight, bias)`` of the norm this block begins with, if the pass that makes the residual before it may
+        also make the rows this block's mixer reads (``forward(..., pre=)`` then takes them); else None."""
+        return self.norm1.spec() if hasattr(self.norm1, "spec") else None
 
     def forward(self, ctx, x, cache: Optional[LayerCache], pre=None, emit=None):
         """``pre``: the rows this block's mixer reads, made by the block before; ``emit``: the ``entry_rows`` of the block
@@ -241,7 +242,7 @@ class SandwichBlock(Block):
             self.norm1b.add_normed(ctx, made, x, slices=slices, then=emit, rounded=handed)
             return handed
         rows = ctx.buffer("h", (n, width), ctx.dtype)
-        self.norm1b.add_normed(ctx, made, x, slices=slices, then=self.norm2, rounded=rows)
+        self.norm1b.add_normed(ctx, made, x, slices=slices, then=self.norm2.spec(), rounded=rows)
         made, slices = self.ffn.forward(ctx, rows, y, store=True) or (y, 1)
         self.norm2b.add_normed(ctx, made, x, slices=slices, then=emit, rounded=handed)
         return handed

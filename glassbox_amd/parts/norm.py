@@ -123,7 +123,7 @@ class TanhNorm(Norm):
         """x = norm(x) on float32 rows (an embedding's output)."""
         ops.tanh_norm(x, self.alpha, self.weight, self.bias, x)
 
-    def add_normed(self, ctx, y, x, slices: int = 1, then: Optional["TanhNorm"] = None, rounded=None) -> None:
-        """x += norm(y) (both float32; ``slices`` > 1: y is the sum of that many pieces); with ``then`` and ``rounded``:
-        rounded = then(new x)."""
-        ops.tanh_norm_add(x, y, self.spec(), slices=slices, then=then.spec() if then is not None else None, h=rounded)
+    def add_normed(self, ctx, y, x, slices: int = 1, then: Optional[tuple] = None, rounded=None) -> None:
+        """x += norm(y) (both float32; ``slices`` > 1: y is the sum of that many pieces); with ``then`` (the ``spec()`` of
+        the norm that reads x next) and ``rounded``: rounded = that norm of the new x."""
+        ops.tanh_norm_add(x, y, self.spec(), slices=slices, then=then, h=rounded)

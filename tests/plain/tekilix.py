@@ -147,28 +147,33 @@ def attend(q, k, v, scale: float, cap: float, mask, sink) -> torch.Tensor:
     return torch.einsum("hij,jhd->ihd", softmax_with_sink(s, mask, sink), vh)
 
 
-def attention(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact) -> torch.Tensor:
-    """Biased projections; one RMS norm over all of q (and of k) before the heads are cut; neighbouring pairs turn;
-    capped scores; a sink of score 0; one sigmoid gate a head."""
+def attention_heads(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact, positions=None):
+    """q [T, H, dk], k [T, G, dk], v [T, G, dv] of the mixer ``attention`` as its scores and sums read them."""
     T = h.shape[0]
     H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    pos = torch.arange(T)
+    pos = torch.arange(T) if positions is None else positions
     q = rnd(h @ w[pre + "q"].T + w[pre + "q.b"])
     k = rnd(h @ w[pre + "k"].T + w[pre + "k.b"])
     v = rnd(h @ w[pre + "v"].T + w[pre + "v.b"]).view(T, G, dv)
     q = (unit_rms(q, eps) * w[pre + "q.norm"]).view(T, H, dk)
     k = (unit_rms(k, eps) * w[pre + "k.norm"]).view(T, G, dk)
-    q, k = rnd(rotate(q, pos, m.get("rot"), True)), rnd(rotate(k, pos, m.get("rot"), True))
+    return rnd(rotate(q, pos, m.get("rot"), True)), rnd(rotate(k, pos, m.get("rot"), True)), v
+
+
+def attention(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact) -> torch.Tensor:
+    """Biased projections; one RMS norm over all of q (and of k) before the heads are cut; neighbouring pairs turn;
+    capped scores; a sink of score 0; one sigmoid gate a head."""
+    T = h.shape[0]
+    H, dv = m["heads"], m["vdim"]
+    q, k, v = attention_heads(w, pre, m, eps, h, rnd)
     chunk = (m.get("mask") or {"size": 0})["size"]
     o = attend(q, k, v, m["scale"], m.get("softcap") or 0.0, visible(T, chunk), torch.zeros(H, dtype=F64))
-    gate = torch.sigmoid(h @ w[pre + "g"].T)                 # [T, H]
+    gate = torch.sigmoid(rnd(h @ w[pre + "g"].T))                 # [T, H]
     return rnd((o * gate[:, :, None]).reshape(T, H * dv)) @ w[pre + "o"].T
 
 
-def attention_2(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact) -> torch.Tensor:
-    """No biases; q and k pass a short convolution over time; the values are the convolved keys; an RMS norm of every
-    head with one weight for all heads; halves of the rotated channels pair up; a learned sink a head; a sigmoid gate
-    on every channel of the heads."""
+def attention_2_heads(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact):
+    """q [T, H, dk], k [T, G, dk], v [T, G, dk] of the mixer ``attention_2`` (whole sequences from position 0)."""
     T = h.shape[0]
     H, G, dk = m["heads"], m["kv_heads"], m["dim"]
     pos = torch.arange(T)
@@ -178,7 +183,16 @@ def attention_2(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact) ->
     v = rnd(k).view(T, G, dk)
     q = unit_rms(q.view(T, H, dk), eps) * w[pre + "q.norm"]
     k = unit_rms(k.view(T, G, dk), eps) * w[pre + "k.norm"]
-    q, k = rnd(rotate(q, pos, m.get("rot"), False)), rnd(rotate(k, pos, m.get("rot"), False))
+    return rnd(rotate(q, pos, m.get("rot"), False)), rnd(rotate(k, pos, m.get("rot"), False)), v
+
+
+def attention_2(w, pre: str, m: dict, eps: float, h: torch.Tensor, rnd=exact) -> torch.Tensor:
+    """No biases; q and k pass a short convolution over time; the values are the convolved keys; an RMS norm of every
+    head with one weight for all heads; halves of the rotated channels pair up; a learned sink a head; a sigmoid gate
+    on every channel of the heads."""
+    T = h.shape[0]
+    H, dk = m["heads"], m["dim"]
+    q, k, v = attention_2_heads(w, pre, m, eps, h, rnd)
     chunk = (m.get("mask") or {"size": 0})["size"]
     o = attend(q, k, v, m["scale"], 0.0, visible(T, chunk), w[pre + "sink"])
     gate = torch.sigmoid(rnd(h @ w[pre + "g"].T))            # [T, H dk]
@@ -208,10 +222,35 @@ def route(z: torch.Tensor, correction: torch.Tensor, top: int, groups: Optional[
     return ids, torch.gather(s, 1, ids)
 
 
-def experts(w, pre: str, mlp: dict, x: torch.Tensor, rnd=exact) -> torch.Tensor:
+def route_margin(z: torch.Tensor, correction: torch.Tensor, top: int, groups: Optional[dict]) -> torch.Tensor:
+    """[T]: by how much a token's choice is clear: the smallest gap between a pick score that decided for an expert (or a
+    group) and the best one that lost; infinite where nothing lost.  A token whose margin is below what rounding moves
+    the scores by may go to other experts in an engine that rounds."""
+    s = torch.softmax(z, -1)
+    pick = s + correction
+    T, E = z.shape
+    margin = torch.full((T,), float("inf"), dtype=z.dtype)
+    if groups:
+        size = E // groups["count"]
+        best = pick.view(T, groups["count"], size).max(-1).values.sort(-1, descending=True).values
+        if groups["keep"] < groups["count"]:
+            margin = best[:, groups["keep"] - 1] - best[:, groups["keep"]]
+        kept = torch.zeros(T, groups["count"], dtype=torch.bool)
+        kept.scatter_(1, torch.topk(pick.view(T, groups["count"], size).max(-1).values, groups["keep"], dim=-1).indices, True)
+        pick = pick.masked_fill(~kept.repeat_interleave(size, 1), float("-inf"))
+    ordered = pick.sort(-1, descending=True).values
+    if top < E:
+        gap = ordered[:, top - 1] - ordered[:, top]
+        margin = torch.minimum(margin, torch.where(torch.isinf(ordered[:, top]), torch.full_like(gap, float("inf")), gap))
+    return margin
+
+
+def experts(w, pre: str, mlp: dict, x: torch.Tensor, rnd=exact, margins: Optional[list] = None) -> torch.Tensor:
     r = mlp["router"]
     z = x @ w[pre + "router"].T
     ids, weights = route(z, w[pre + "correction"], r["top"], r.get("groups"))
+    if margins is not None:
+        margins.append(route_margin(z, w[pre + "correction"], r["top"], r.get("groups")))
     y = torch.zeros_like(x)
     for e in range(r["experts"]):
         chosen = (ids == e)
@@ -238,8 +277,9 @@ def embed(cfg: dict, w, tokens: List[int]) -> torch.Tensor:
 
 
 def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], coarse: bool = False,
-            tap: Optional[list] = None) -> torch.Tensor:
-    """Logits [T, vocab] of one whole sequence.  ``tap`` receives the residual after every layer."""
+            tap: Optional[list] = None, margins: Optional[list] = None) -> torch.Tensor:
+    """Logits [T, vocab] of one whole sequence.  ``tap`` receives the residual after every layer, ``margins`` every
+    router's ``route_margin``."""
     rnd = bf16 if coarse else exact
     eps = cfg["norm"]["eps"]
     x = embed(cfg, w, tokens)
@@ -255,7 +295,7 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], coarse: bo
         x = x + tanh_norm(w, name + "norm1b", y)
         if layer.get("mlp") is not None:
             h = rnd(tanh_norm(w, name + "norm2", x))
-            x = x + tanh_norm(w, name + "norm2b", experts(w, name + "mlp.", layer["mlp"], h, rnd))
+            x = x + tanh_norm(w, name + "norm2b", experts(w, name + "mlp.", layer["mlp"], h, rnd, margins))
         if tap is not None:
             tap.append(x.clone())
     return rnd(tanh_norm(w, "final.norm", x)) @ w["embed"].T * cfg["logit_scale"]

@@ -1,0 +1,680 @@
+"""Tekilix on the device: each mechanism's kernels against the plain implementation, then whole models under every
+way of cutting requests into steps, and generation through the entry points."""
+from __future__ import annotations
+
+import copy
+import json
+import math
+import os
+import subprocess
+import sys
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+from plain import tekilix as pt
+from tekilix_cases import CASES, folder_of, rounded
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+DEV = "cuda:0"
+
+
+def _dev(t, dtype=torch.float32):
+    return t.to(dtype).to(DEV).contiguous()
+
+
+def _i32(values):
+    return torch.tensor(list(values), dtype=torch.int32, device=DEV)
+
+
+def _step_ctx(rows, slots):
+    """The tables of a step whose requests bring ``rows`` = [(request, first position, end position)], in that order."""
+    lens = [b - a for _, a, b in rows]
+    starts = np.cumsum([0] + lens)[:-1]
+    tok_seq = [s for s, n in enumerate(lens) for _ in range(n)]
+    return SimpleNamespace(q_start=_i32(starts), q_len=_i32(lens), pos0=_i32(a for _, a, _ in rows), tok_seq=_i32(tok_seq),
+                           state_slots=_i32(slots[r] for r, _, _ in rows), num_seqs=len(rows),
+                           host={"max_q_len": max(lens), "n_decode": sum(1 for n in lens if n == 1)})
+
+
+def _pool(T, P, G, hc, dtype, seed=0):
+    """Pages for one request of T tokens, handed out in a shuffled order among pages that hold garbage."""
+    from glassbox_amd import ops
+    n_pages = -(-T // P)
+    order = np.random.RandomState(seed).permutation(n_pages + 3)[:n_pages].tolist()
+    slots = [order[p // P] * P + p % P for p in range(T)]
+    k_pages = torch.full(ops.key_pages_shape(n_pages + 3, G, P, hc), 77.0, dtype=dtype, device=DEV)
+    v_pages = torch.full((n_pages + 3, G, hc, P), -55.0, dtype=dtype, device=DEV)
+    return order, slots, k_pages, v_pages
+
+
+# ------------------------------------------------------------------------------------------ the bounded norm
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_the_bounded_norm_of_rows_of_picked_rows_in_place_and_on_the_way_into_the_residual(dtype):
+    from glassbox_amd import ops
+    torch.manual_seed(4)
+    tol = 2e-6 if dtype == torch.float32 else 1e-2
+    for n, d in ((5, 64), (70, 50), (3, 7), (130, 320)):
+        x = torch.randn(n, d, dtype=F64) * 2
+        w = {"n": torch.randn(d, dtype=F64), "n.b": torch.randn(d, dtype=F64) * 0.3, "n.alpha": torch.tensor(0.7, dtype=F64),
+             "m": torch.rand(d, dtype=F64) + 0.5, "m.b": torch.randn(d, dtype=F64), "m.alpha": torch.tensor(1.9, dtype=F64)}
+        spec = lambda k: (_dev(w[k + ".alpha"].reshape(1)), _dev(w[k]), _dev(w[k + ".b"]))
+        want = pt.tanh_norm(w, "n", x.float().to(F64))
+        out = torch.empty(n, d + 3, dtype=dtype, device=DEV)[:, :d]
+        ops.tanh_norm(_dev(x), *spec("n"), out)
+        assert (out.cpu().to(F64) - want).abs().max() < tol * float(want.abs().max())
+        rows = [n - 1, 0, n // 2]
+        picked = torch.empty(3, d, dtype=dtype, device=DEV)
+        ops.tanh_norm(_dev(x), *spec("n"), picked, _i32(rows))
+        assert torch.equal(picked, out[rows])
+        if dtype == torch.float32:
+            same = _dev(x)
+            ops.tanh_norm(same, *spec("n"), same)
+            assert torch.equal(same, out)
+        # x += n(y), y in three pieces, and the rows the next norm makes of the new x
+        pieces = torch.randn(3, n, d, dtype=F64).float()
+        res = _dev(x)
+        nxt = torch.empty(n, d, dtype=dtype, device=DEV)
+        ops.tanh_norm_add(res, _dev(pieces), spec("n"), slices=3, then=spec("m"), h=nxt)
+        y = (pieces[0] + pieces[1]) + pieces[2]
+        new = x.float().to(F64) + pt.tanh_norm(w, "n", y.to(F64))
+        assert (res.cpu().to(F64) - new).abs().max() < 2e-6 * float(new.abs().max())
+        after = pt.tanh_norm(w, "m", res.cpu().to(F64))
+        assert (nxt.cpu().to(F64) - after).abs().max() < tol * float(after.abs().max())
+        alone = _dev(x)
+        ops.tanh_norm_add(alone, _dev(y), spec("n"))
+        assert torch.equal(alone, res)
+
+
+# ------------------------------------------------------------------------------------------ the heads' preparation
+def _mixer_weights(kind, m, width, seed):
+    torch.manual_seed(seed)
+    H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    r = lambda *s: torch.randn(*s, dtype=F64)
+    w = {"x.q": r(H * dk, width) * 0.3, "x.k": r(G * dk, width) * 0.3}
+    if kind == "attention":
+        w.update({"x.v": r(G * dv, width) * 0.3, "x.q.b": r(H * dk), "x.k.b": r(G * dk), "x.v.b": r(G * dv),
+                  "x.q.norm": r(H * dk) + 1.0, "x.k.norm": r(G * dk) + 1.0})
+    else:
+        w.update({"x.q.norm": r(dk) + 1.0, "x.k.norm": r(dk) + 1.0})
+        if m.get("conv"):
+            w.update({"x.q.conv": r(H * dk, m["conv"]) * 0.6, "x.k.conv": r(G * dk, m["conv"]) * 0.6})
+    return w
+
+
+HEAD_CASES = [
+    ("attention", {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 16, "rot": {"dims": 8, "base": 100.0}}),
+    ("attention", {"heads": 2, "kv_heads": 1, "dim": 6, "vdim": 10, "rot": {"dims": 6, "base": 50.0}}),
+    ("attention", {"heads": 3, "kv_heads": 3, "dim": 144, "vdim": 64}),
+    ("attention_2", {"heads": 4, "kv_heads": 1, "dim": 16, "vdim": 16, "conv": 4,
+                     "rot": {"dims": 16, "base": 1000.0, "scaling": {"factor": 8.0, "original": 64, "fast": 4.0, "slow": 1.0}}}),
+    ("attention_2", {"heads": 3, "kv_heads": 3, "dim": 10, "vdim": 10, "conv": 2, "rot": {"dims": 2, "base": 20.0}}),
+    ("attention_2", {"heads": 2, "kv_heads": 2, "dim": 40, "vdim": 40, "conv": 8, "rot": {"dims": 12, "base": 300.0}}),
+    ("attention_2", {"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 32, "conv": 1}),
+    ("attention_2", {"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 32, "rot": {"dims": 32, "base": 7.0}}),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind, m", HEAD_CASES)
+def test_heads_prepared_in_portions_of_a_batch(kind, m, dtype):
+    """Three requests whose tokens come in four steps of unequal portions (single tokens, portions shorter than the
+    convolution, long ones; the first and third steps bring single tokens only, so the kernel moves the slots on
+    itself) into pages and slots that hold garbage: query, key and value heads against the plain functions on whole
+    sequences, the pages' contents, and the slots after every step."""
+    from glassbox_amd import ops
+    from glassbox_amd.parts.attention import cache_head_cols
+    from glassbox_amd.parts.rotary import Rotary
+    width, eps, P = 40, 1e-5, 16
+    H, G, dk, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    w = _mixer_weights(kind, m, width, seed=H * dk)
+    f = lambda t: t.to(dtype).to(F64)
+    lens = {0: 23, 1: 3, 2: 9}
+    cuts = {0: (1, 20, 1, 1), 1: (1, 1, 0, 1), 2: (1, 2, 1, 5)}
+    state_slots = {0: 2, 1: 0, 2: 3}
+    hidden = {r: torch.randn(T, width, dtype=F64) for r, T in lens.items()}
+    proj_names = ["x.q", "x.k"] + (["x.v"] if kind == "attention" else [])
+    proj = {r: f(torch.cat([h @ w[n].T for n in proj_names], 1)) for r, h in hidden.items()}   # what the product leaves
+    if kind == "attention":
+        # (the kernel starts from the projections as the product left them, rounded: so do the plain steps here)
+        def heads_of(r):
+            T = lens[r]
+            q = proj[r][:, :H * dk] + w["x.q.b"]
+            k = proj[r][:, H * dk:(H + G) * dk] + w["x.k.b"]
+            v = (proj[r][:, (H + G) * dk:] + w["x.v.b"]).view(T, G, dv)
+            q = (pt.unit_rms(q, eps) * w["x.q.norm"]).view(T, H, dk)
+            k = (pt.unit_rms(k, eps) * w["x.k.norm"]).view(T, G, dk)
+            pos = torch.arange(T)
+            return pt.rotate(q, pos, m.get("rot"), True), pt.rotate(k, pos, m.get("rot"), True), v
+    else:
+        def heads_of(r):
+            T = lens[r]
+            q, k = proj[r][:, :H * dk], proj[r][:, H * dk:]
+            if m.get("conv"):
+                q, k = pt.causal_conv(q, w["x.q.conv"]), pt.causal_conv(k, w["x.k.conv"])
+            v = k.view(T, G, dk)
+            q = pt.unit_rms(q.view(T, H, dk), eps) * w["x.q.norm"]
+            k = pt.unit_rms(k.view(T, G, dk), eps) * w["x.k.norm"]
+            pos = torch.arange(T)
+            return pt.rotate(q, pos, m.get("rot"), False), pt.rotate(k, pos, m.get("rot"), False), v
+    want = {r: heads_of(r) for r in lens}
+    hc = cache_head_cols(dk, dv)
+    taps = m.get("conv", 0) if kind == "attention_2" else 0
+    channels = (H + G) * dk
+    state = torch.full((5, taps - 1, channels), 55.0, device=DEV) if taps > 1 else None
+    bias = _dev(torch.cat([w["x.q.b"], w["x.k.b"], w["x.v.b"]])) if kind == "attention" else None
+    wconv = _dev(torch.cat([w["x.q.conv"], w["x.k.conv"]], 0)) if taps else None
+    rot = m.get("rot")
+    rotary = Rotary(rot["dims"], rot["base"], tuple(rot["scaling"][k] for k in ("factor", "original", "fast", "slow"))
+                    if rot.get("scaling") else None) if rot else None
+    pools = {r: _pool(T, P, G, hc, dtype, seed=r) for r, T in lens.items()}
+    tol = 3e-5 if dtype == torch.float32 else 3e-2
+    done = {r: 0 for r in lens}
+    for step in range(4):
+        rows = [(r, done[r], done[r] + cuts[r][step]) for r in lens if cuts[r][step]]
+        rows.sort(key=lambda x: x[2] - x[1] > 1)
+        ctx = _step_ctx(rows, state_slots)
+        positions = [p for r, a, b in rows for p in range(a, b)]
+        n = len(positions)
+        cos = sin = None
+        if rotary is not None:
+            cos, sin = torch.empty(n, rot["dims"] // 2, device=DEV), torch.empty(n, rot["dims"] // 2, device=DEV)
+            ops.rope_table(_i32(positions), torch.from_numpy(rotary.inv_host).to(DEV), cos, sin)
+        # one pool of pages a request: the step's rows of each request are prepared with that request's pages
+        x = torch.cat([proj[r][a:b] for r, a, b in rows], 0)
+        x = _dev(torch.cat([x, torch.full((n, 5), 9.0, dtype=F64)], 1), dtype)[:, :x.shape[1] + 3]   # gates' columns behind
+        heads = torch.full((n, (H + 2 * G) * hc), 3.0, dtype=dtype, device=DEV)
+        # the kernel writes every row's keys and values into one pool: lay the requests' pools side by side
+        n_pages = [pools[r][2].shape[0] for r in lens]
+        base = {r: sum(n_pages[:i]) for i, r in enumerate(lens)}
+        if step == 0:
+            k_all = torch.cat([pools[r][2] for r in lens], 0).contiguous()
+            v_all = torch.cat([pools[r][3] for r in lens], 0).contiguous()
+        slots = [base[r] * P + pools[r][1][p] for r, a, b in rows for p in range(a, b)]
+        ops.qk_heads(x, ctx, heads, hc, H, G, dk, dv, eps, kind == "attention", _dev(w["x.q.norm"]), _dev(w["x.k.norm"]), bias=bias,
+                     wconv=wconv, state=state, cos=cos, sin=sin, rot=rot["dims"] if rot else 0,
+                     magnitude=rotary.magnitude if rotary is not None else 1.0, neighbours=kind == "attention",
+                     tied=kind == "attention_2", slots=_i32(slots), k_pages=k_all, v_pages=v_all)
+        got, at = heads.cpu().to(F64).view(n, H + 2 * G, hc), 0
+        stored_k = ops.unpack_keys(k_all).cpu().to(F64)
+        for r, a, b in rows:
+            q, k, v = want[r]
+            scale = max(1.0, float(q.abs().max()), float(k.abs().max()), float(v.abs().max()))
+            part = got[at:at + b - a]
+            assert (part[:, :H, :dk] - q[a:b]).abs().max() < tol * scale, (step, r, "q")
+            assert (part[:, H:H + G, :dk] - k[a:b]).abs().max() < tol * scale, (step, r, "k")
+            assert (part[:, H + G:, :dv] - v[a:b]).abs().max() < tol * scale, (step, r, "v")
+            assert float(part[:, :H + G, dk:].abs().max() if hc > dk else 0.0) == 0.0
+            assert float(part[:, H + G:, dv:].abs().max() if hc > dv else 0.0) == 0.0
+            for p in (a, b - 1):
+                page, slot = base[r] + pools[r][0][p // P], p % P
+                assert torch.equal(stored_k[page, :, slot], part[p - a, H:H + G])
+                assert torch.equal(v_all[page, :, :, slot].cpu().to(F64), part[p - a, H + G:])
+            at += b - a
+            done[r] = b
+            if state is not None:
+                kept = state[state_slots[r]].cpu().to(F64)
+                for i in range(taps - 1):
+                    p = b - (taps - 1) + i
+                    if p >= 0:
+                        assert torch.equal(kept[i], proj[r][p, :channels]), (step, r, i)
+    if state is not None:
+        assert torch.all(state[1] == 55.0) and torch.all(state[4] == 55.0)   # nobody else's slot was touched
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gates_of_heads_and_of_channels(dtype):
+    from glassbox_amd import ops
+    torch.manual_seed(2)
+    f = lambda t: t.to(dtype).to(F64)
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    for n, H, hc, V in ((6, 4, 32, 16), (65, 3, 48, 48), (2, 2, 136, 40), (9, 5, 16, 10)):
+        att = f(torch.randn(n, H, hc, dtype=F64))
+        for per_head in (True, False):
+            cols = H if per_head else H * V
+            wide = f(torch.randn(n, 7 + cols + 3, dtype=F64) * 3)
+            gate = wide[:, 7:7 + cols]
+            out = torch.empty(n, H * V, dtype=dtype, device=DEV)
+            ops.gate_rows(_dev(att.reshape(n, H * hc), dtype), hc, _dev(wide, dtype)[:, 7:7 + cols], out, H, V, per_head)
+            g = torch.sigmoid(gate).view(n, H, 1 if per_head else V)
+            want = (att[:, :, :V] * g).reshape(n, H * V)
+            assert (out.cpu().to(F64) - want).abs().max() < tol * float(want.abs().max())
+
+
+# ------------------------------------------------------------------------------------------ attention itself
+def _attention_inputs(T, H, G, hc, dk, dv, dtype, seed):
+    """Queries and keys of one request at positions 0 .. T - 1 with a few keys that would each dominate the softmax of a
+    later query if it were visible: the query of position i is, beside noise, ``pull`` times the key that stands
+    ``back[i]`` positions before it."""
+    g = torch.Generator().manual_seed(seed)
+    f = lambda t: t.to(dtype).to(F64)
+    q = torch.randn(T, H, hc, generator=g, dtype=F64) * 0.3
+    k = torch.randn(T, G, hc, generator=g, dtype=F64) * 0.3
+    v = torch.randn(T, G, hc, generator=g, dtype=F64)
+    q[..., dk:], k[..., dk:], v[..., dv:] = 0.0, 0.0, 0.0
+    return f(q), f(k), f(v)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H, G, dk, dv, chunk, softcap, sink", [
+    (4, 2, 32, 32, 24, 4.0, "zero"), (2, 1, 64, 64, 200, 0.0, "learned"), (6, 1, 16, 48, 7, 30.0, "zero"),
+    (2, 2, 136, 136, 64, 0.0, "learned"), (3, 3, 40, 24, 0, 2.0, None), (8, 2, 96, 96, 50, 0.0, "zero")])
+def test_attention_at_the_edges_of_runs_with_sinks_and_capped_scores(dtype, H, G, dk, dv, chunk, softcap, sink):
+    """One request of 700 tokens.  Queries are built so that the first key of their own run, the last key of the run
+    before, a key far back inside the run and one far back outside it would each take most of the softmax if it were
+    visible; sinks large enough to take a visible share; scores far into the cap.  The plain kernel whole, in portions
+    and token by token with a workgroup a chunk of keys, and the matrix-core kernels for portions and single tokens,
+    against the plain functions."""
+    from glassbox_amd import ops
+    from glassbox_amd.parts.attention import cache_head_cols, paged_attention
+    from glassbox_amd.engine.context import Workspace
+    T, P, scale = 700, 16, 0.4
+    hc = cache_head_cols(dk, dv)
+    q, k, v = _attention_inputs(T, H, G, hc, dk, dv, dtype, seed=H * dk + chunk)
+    group = H // G
+    run = chunk if chunk else T
+    for i in range(40, T, 7):
+        start = i - i % run
+        target = [start, start - 1, max(start, i - 150), i - 300, i - 1][(i // 7) % 5]
+        if target < 0:
+            continue
+        for h in range(H):
+            q[i, h] = q[i, h] + 6.0 * k[target, h // group] / (scale * float((k[target, h // group] ** 2).sum()) ** 0.5)
+    q = q.to(dtype).to(F64)
+    sinks = None if sink is None else torch.zeros(H, dtype=F64) if sink == "zero" else torch.linspace(-1.0, 3.0, H, dtype=F64)
+    s = pt.capped(torch.einsum("ihd,jhd->hij", q, k.repeat_interleave(group, 1)) * scale, softcap)
+    mask = pt.visible(T, chunk)
+    if sinks is None:
+        p = torch.softmax(s.masked_fill(~mask[None], float("-inf")), -1)
+    else:
+        p = pt.softmax_with_sink(s, mask, sinks)
+    want = torch.einsum("hij,jhd->ihd", p, v.repeat_interleave(group, 1)).reshape(T, H * hc)
+    if chunk and chunk < 300:
+        assert float(p[:, 40:, :].max(-1).values.min()) < 0.9 < float(p.max())   # some queries found their key, others did not
+    order, slots, k_pages, v_pages = _pool(T, P, G, hc, dtype, seed=1)
+    heads = _dev(torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1), dtype)
+    ops.rope_store(heads, None, None, _i32(slots), k_pages, v_pages, H, G, hc, rotate=False)
+    table = _i32(order).view(1, -1)
+    sink_dev = _dev(sinks) if sinks is not None else None
+    tol = 3e-5 if dtype == torch.float32 else 3e-2
+    limit = tol * max(1.0, float(want.abs().max()))
+    out = torch.empty(T, H * hc, dtype=dtype, device=DEV)
+    ops.attention_plain(heads[:, :H * hc], out, _i32(range(T)), _i32([0] * T), table, k_pages, v_pages, H, scale, 0,
+                        chunk=chunk, softcap=softcap, sinks=sink_dev)
+    assert (out.cpu().to(F64) - want).abs().max() < limit, "plain kernel, whole"
+    # a workgroup a chunk of 256 keys, merged by a second kernel: the same bits
+    rows = list(range(T - 9, T))
+    floats = ops.attention_plain_split_floats(len(rows), H, hc, P, T)
+    if floats:
+        split = torch.empty(len(rows), H * hc, dtype=dtype, device=DEV)
+        ops.attention_plain(heads[rows, :H * hc], split, _i32(rows), _i32([0] * len(rows)), table, k_pages, v_pages, H, scale, 0,
+                            workspace=torch.empty(floats, device=DEV), max_context=T, chunk=chunk, softcap=softcap, sinks=sink_dev)
+        assert torch.equal(split, out[rows])
+    if dtype != torch.bfloat16 or not ops.tuned_attention_supports(k_pages, H, 0, 0):
+        return
+    # the matrix-core kernels through the mixers' own entry: single tokens at the ends of runs, portions of any cut
+    cache = SimpleNamespace(k_pages=k_pages, v_pages=v_pages, group=0)
+    ws = Workspace(torch.device(DEV))
+    singles = [[p] for p in (T - 1, max(chunk, 1), max(chunk, 1) - 1, 2 * run - 1 if 2 * run <= T else T - 2, 0, 300)]
+    steps = [singles, [list(range(0, 311))], [list(range(311, 313))], [list(range(313, T))], [[T - 1], list(range(100, 430))],
+             [[5], [T - 2], list(range(run - 1, run + 40)) if run + 40 <= T else list(range(20, 90)), list(range(3, 5))]]
+    for rows in steps:   # the rows of a step: single tokens first, then portions (each as a request of its own)
+        flat = [p for r in rows for p in r]
+        lens = [len(r) for r in rows]
+        n_dec = sum(1 for l in lens if l == 1)
+        ctx = SimpleNamespace(dtype=torch.bfloat16, tuned=True, n=len(flat), num_seqs=len(rows),
+                              positions=_i32(flat), tok_seq=_i32(s for s, l in enumerate(lens) for _ in range(l)),
+                              tables=[table.expand(len(rows), -1).contiguous()],
+                              q_start=_i32(np.cumsum([0] + lens)[:-1]), q_len=_i32(lens), pos0=_i32(r[0] for r in rows),
+                              host={"n_decode": n_dec, "max_q_len": max(lens), "max_context": max(flat) + 1},
+                              buffer=ws.buffer)
+        got = torch.empty(len(flat), H * hc, dtype=dtype, device=DEV)
+        paged_attention(ctx, heads[flat, :H * hc].contiguous(), got, cache, H, scale, 0, 0, chunk, softcap, sink_dev)
+        assert (got.cpu().to(F64) - want[flat]).abs().max() < limit, ("matrix-core kernels", lens[:4], flat[:4])
+
+
+# ------------------------------------------------------------------------------------------ the router and the experts
+@pytest.mark.parametrize("E, top, groups", [(6, 2, (3, 2)), (8, 4, (4, 3)), (16, 3, (4, 2)), (12, 5, (4, 4)), (4, 4, None), (5, 3, None),
+                                            (3, 1, None), (4, 2, (1, 1)), (64, 6, (8, 3)), (130, 16, (13, 4))])
+def test_the_router_scores_by_softmax_and_chooses_within_the_best_groups(E, top, groups):
+    from glassbox_amd import ops
+    torch.manual_seed(E + top)
+    n = 301
+    z = torch.randn(n, E + 2) * 2
+    corr = torch.randn(E) * 0.1
+    z[7, :E] = -50.0          # nearly all weight on one expert: the others' picks are their corrections, which may be negative
+    z[7, 1] = 50.0
+    ids_w, wts_w = pt.route(z[:, :E].to(F64), corr.to(F64), top, {"count": groups[0], "keep": groups[1]} if groups else None)
+    combine = torch.empty(n, E + 1, device=DEV)
+    ids, wts = torch.empty(n, top, dtype=torch.int32, device=DEV), torch.empty(n, top, device=DEV)
+    ops.moe_route(_dev(z)[:, :E], E, _dev(corr), top, 1.0, "whole", combine, ids, wts, softmax=True, renorm=False,
+                  groups=groups[0] if groups else 0, keep_groups=groups[1] if groups else 0)
+    s = torch.softmax(z[:, :E].to(F64), -1)
+    pick = s + corr.to(F64)
+    margins = []
+    for t in range(n):
+        mine, theirs = set(ids[t].tolist()), set(ids_w[t].tolist())
+        if mine != theirs:   # only where two picks are as good as equal in 32-bit
+            a, b = (mine - theirs).pop(), (theirs - mine).pop()
+            assert abs(float(pick[t, a] - pick[t, b])) < 1e-6, (t, mine, theirs)
+            continue
+        margins.append(t)
+        for kk in range(top):
+            e = int(ids[t, kk])
+            assert abs(float(wts[t, kk]) - float(s[t, e])) < 1e-6
+        row = combine[t].cpu().to(F64)
+        assert float(row[E]) == 1.0 and abs(float(row[:E].sum()) - float(wts[t].sum())) < 1e-5
+        assert int((row[:E] != 0).sum()) <= top
+    assert len(margins) > n - 5
+    if groups and groups[1] < groups[0]:
+        size = E // groups[0]
+        assert all(len({int(e) // size for e in ids[t].tolist()}) <= groups[1] for t in range(n))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_squared_relu_units_with_and_without_weights(dtype):
+    from glassbox_amd import ops
+    torch.manual_seed(5)
+    E, ff, shared, n = 5, 12, 20, 37
+    z = (torch.randn(n, E * ff + shared, dtype=F64) * 2).to(dtype).to(F64)
+    combine = torch.rand(n, E + 1, dtype=F64).float().to(F64)
+    combine[:, 1] = 0.0
+    act = torch.empty(n, E * ff + shared, dtype=dtype, device=DEV)
+    ops.moe_relu2_units(_dev(z, torch.float32), _dev(combine), act, E, ff)
+    wcol = torch.cat([combine[:, :E].repeat_interleave(ff, 1), combine[:, E:].expand(n, shared)], 1)
+    want = torch.relu(z) ** 2 * wcol
+    tol = 1e-6 if dtype == torch.float32 else 1e-2
+    assert (act.cpu().to(F64) - want).abs().max() < tol * float(want.abs().max())
+    assert float(act[:, ff:2 * ff].abs().max()) == 0.0
+    same = _dev(z, dtype)
+    ops.moe_relu2_units(same, None, same, 0, ff)
+    assert (same.cpu().to(F64) - torch.relu(z) ** 2).abs().max() < tol * float(want.abs().max()) * 4
+
+
+def test_experts_on_their_own_tokens_against_every_expert_on_every_token():
+    """The two ways through a step of the routed feed-forward (few rows: every expert on every token, zeros for the ones
+    not chosen; many rows: sorted by expert) against the plain sum, with one expert's down matrix a hundred times the
+    others', so that a token sent to a wrong expert or weighted wrongly shows."""
+    from glassbox_amd.engine.context import Workspace
+    from glassbox_amd.parts.moe import RoutedExperts
+    torch.manual_seed(8)
+    d, E, top, ff, shared = 64, 8, 2, 16, 32
+    part = RoutedExperts(d, E, top, ff, 1.0, shared, correction=True, scoring="softmax", renorm=False, groups=(4, 3), unit="relu2",
+                         shared_gate=False)
+    w = {n: torch.randn(s.shape, dtype=F64) * (0.1 if len(s.shape) == 2 else 0.05) for n, s in part.tensor_specs().items()}
+    w["router"] = w["router"] * 8
+    w["e3.down"] = w["e3.down"] * 100
+    w = {n: t.to(torch.bfloat16).to(F64) if t.dim() == 2 else t for n, t in w.items()}
+    part.load({n: _dev(t, torch.bfloat16 if t.dim() == 2 else torch.float32) for n, t in w.items()})
+    mlp = {"router": {"experts": E, "top": top, "groups": {"count": 4, "keep": 3}}, "shared": {"ff": shared}}
+    ws = Workspace(torch.device(DEV))
+    for n in (5, 300):
+        h = (torch.randn(n, d, dtype=F64)).to(torch.bfloat16).to(F64)
+        want = pt.experts({"m." + k: v for k, v in w.items()}, "m.", mlp, h, rnd=pt.bf16)
+        ctx = SimpleNamespace(dtype=torch.bfloat16, buffer=ws.buffer, tuned=True, fuse_norms=True)
+        y = torch.full((n, d), 5.0, device=DEV)
+        assert part.routed(ctx, n) == (n > 64)
+        part.forward(ctx, _dev(h, torch.bfloat16), y, store=True)
+        err = (y.cpu().to(F64) - want).abs().max(1).values
+        assert float(err.max()) < 2e-2 * float(want.abs().max()), (n, float(err.max()), float(want.abs().max()))
+        add = torch.ones(n, d, device=DEV)
+        part.forward(ctx, _dev(h, torch.bfloat16), add)
+        assert (add - 1.0 - y).abs().max() < 1e-3 * float(want.abs().max())
+
+
+# ------------------------------------------------------------------------------------------ whole models
+REQUESTS = {"a": 150, "b": 77, "c": 41, "d": 3, "e": 1, "f": 97}
+
+
+def _requests(vocab: int, seed: int = 0):
+    return {r: helpers.random_tokens(vocab, n, seed=seed + n) for r, n in REQUESTS.items()}
+
+
+_ORACLE: dict = {}
+
+
+def _want(folder: str, tokens, dtype: str) -> np.ndarray:
+    key = (folder, tuple(tokens), dtype)
+    if key not in _ORACLE:
+        cfg, w = pt.load_folder(folder)
+        _ORACLE[key] = pt.forward(cfg, rounded(w) if dtype == "bfloat16" else w, list(tokens)).numpy()
+    return _ORACLE[key]
+
+
+def _moved_by_rounding(folder: str, tokens) -> np.ndarray:
+    """How far rounding the activations to bfloat16 moves each position's logits in the plain implementation (root mean
+    square over the vocabulary): what a position's sensitivity to rounding is."""
+    key = (folder, tuple(tokens), "moved")
+    if key not in _ORACLE:
+        cfg, w = pt.load_folder(folder)
+        coarse = pt.forward(cfg, rounded(w), list(tokens), coarse=True).numpy()
+        _ORACLE[key] = np.sqrt(((coarse - _want(folder, tokens, "bfloat16")) ** 2).mean(1))
+    return _ORACLE[key]
+
+
+def _close_calls(folder: str, tokens) -> np.ndarray:
+    """Positions at which some router's choice hangs on less than rounding to bfloat16 moves its scores by: a margin
+    (``route_margin``) below ``ROUTE_TIMES`` times what rounding the activations moved that margin by in the plain
+    implementation itself, or below ``ROUTE_MARGIN``.  There an engine that rounds may send the token to other experts
+    than the plain implementation does, both being right; such positions are left out of the comparison in bfloat16."""
+    key = (folder, tuple(tokens), "margins")
+    if key not in _ORACLE:
+        cfg, w = pt.load_folder(folder)
+        fine, coarse = [], []
+        pt.forward(cfg, rounded(w), list(tokens), margins=fine)
+        pt.forward(cfg, rounded(w), list(tokens), margins=coarse, coarse=True)
+        if not fine:
+            _ORACLE[key] = np.zeros(len(tokens), dtype=bool)
+        else:
+            a, b = torch.stack(fine).clamp(max=1.0), torch.stack(coarse).clamp(max=1.0)
+            _ORACLE[key] = (a < torch.clamp(ROUTE_TIMES * (a - b).abs(), min=ROUTE_MARGIN)).any(0).numpy()
+    return _ORACLE[key]
+
+
+ROUTE_MARGIN, ROUTE_TIMES = 1e-3, 3.0
+
+#: A 32-bit engine is held to helpers.TOL_F32 of the request's largest logit at every position.  A bfloat16 engine is
+#: compared with the plain implementation on the weights it holds by the root mean square of a position's logit
+#: differences: at most 3 times what rounding the activations moves that position in the plain implementation itself, or
+#: 1 % of the request's logits' root mean square where that is more.  One sample of rounding is no sharp bound on
+#: another: a position's movement counts as at least the median over its request; no position may be beyond one and
+#: a half times its limit, and one in fifty beyond the limit itself.
+BF16_TIMES, BF16_FLOOR = 3.0, 1e-2
+
+
+def _check(got, folder, requests, dtype, what):
+    for r, toks in requests.items():
+        want = _want(folder, toks, dtype)
+        if dtype == "float32":
+            tol = helpers.TOL_F32 * max(1.0, float(np.abs(want).max()))
+            bad = helpers.first_bad(got[r], want, tol)
+            assert bad is None, f"{what}, {dtype}, request {r} ({len(toks)} tokens): position {bad[0]} is {bad[1]:.3e} off (limit {tol:.3e})"
+            continue
+        err = np.sqrt(((got[r] - want) ** 2).mean(1))
+        moved = _moved_by_rounding(folder, toks)
+        lim = np.maximum(BF16_TIMES * np.maximum(moved, np.median(moved)), BF16_FLOOR * float(np.sqrt((want ** 2).mean())))
+        close = _close_calls(folder, toks)
+        assert close.sum() <= max(2, len(toks) // 4), f"{close.sum()} of {len(toks)} positions are close calls of a router"
+        err = np.where(close, 0.0, err)
+        # a token that went to other experts has other keys and values in the layers after: the positions behind it
+        # that read them are moved too, by less; they get three times the room
+        lim = np.where(np.cumsum(close) > 0, 3.0 * lim, lim)
+        over = np.nonzero(err > lim)[0]
+        assert over.size <= max(1, len(toks) // 50) and float((err / lim).max()) <= 1.5, (
+            f"{what}, {dtype}, request {r} ({len(toks)} tokens): position {over[0]} is {err[over[0]]:.3e} off "
+            f"(limit {lim[over[0]]:.3e}); {over.size} positions over their limits, worst ratio {(err / lim).max():.2f}")
+
+
+def _poison(engine) -> None:
+    """Garbage in every page and state slot: whatever a request reads, it must have written itself."""
+    for lc in engine.layers:
+        for t in (lc.k_pages, lc.v_pages, lc.state):
+            if t is not None:
+                t.fill_(300.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CASES))
+def test_every_way_of_cutting_requests_into_steps(model_dirs, name, dtype):
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, name)
+    requests = _requests(CASES[name]["vocab"])
+    mixed, peak = helpers.schedule_mixed(requests, seed=3, live=3, tail=20)
+    eng = Engine(folder, dtype=dtype, max_tokens=max(peak, 192), max_seqs=3)
+    _poison(eng)
+    for what, steps in (("whole", helpers.schedule_whole(requests)), ("last tokens one by one", helpers.schedule_tail(requests, 60)),
+                        ("portions", helpers.schedule_chunks(requests)), ("portions of two", None), ("mixed batches", mixed)):
+        if what == "portions of two":
+            steps = helpers.schedule_chunks({r: t for r, t in requests.items() if len(t) < 80}, (2,))
+        got = helpers.replay(eng, steps)
+        _check(got, folder, {r: requests[r] for r in got}, dtype, what)
+        assert eng.cache.num_seqs() == 0 and eng.cache.free_state_slots() == 3
+        assert all(eng.cache.used_pages(g) == 0 for g in range(len(eng.group_keys)))
+        eng.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_long_prompts_whole_and_in_long_portions(model_dirs, name, dtype):
+    """A prompt of 700 tokens: the runs of positions end many times, the stretched frequencies turn far, and the experts
+    are run on their own tokens (many rows)."""
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, name)
+    vocab = CASES[name]["vocab"]
+    requests = {"long": helpers.random_tokens(vocab, 700, seed=23), "short": helpers.random_tokens(vocab, 40, seed=22)}
+    eng = Engine(folder, dtype=dtype, max_tokens=1024, max_seqs=2)
+    _poison(eng)
+    for what, steps in (("whole", helpers.schedule_whole(requests)), ("long portions", helpers.schedule_chunks(requests, (300, 1, 399))),
+                        ("a long portion beside single tokens", [
+                            {"entries": [("short", requests["short"][:39], list(range(39)))], "end": []},
+                            {"entries": [("long", requests["long"], list(range(700))), ("short", requests["short"][39:], [0])],
+                             "end": ["long", "short"]}])):
+        got = helpers.replay(eng, steps)
+        _check(got, folder, requests, dtype, what)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_dirs, dtype):
+    """250 tokens one by one after a prompt of four (runs and pages end many times over; in bfloat16 the steps are
+    replayed from graphs)."""
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, "A")
+    toks = helpers.random_tokens(211, 254, seed=11)
+    steps = helpers.schedule_tail({"x": toks}, 250)
+    eng = Engine(folder, dtype=dtype, max_tokens=320, max_seqs=2)
+    _poison(eng)
+    got = helpers.replay(eng, steps)
+    if dtype == "bfloat16":
+        assert eng.decode_graphs is not None and eng.decode_graphs.replays > 200
+    _check(got, folder, {"x": toks}, dtype, "long decoding")
+    plain = Engine(folder, dtype=dtype, max_tokens=320, max_seqs=2, graph_decode=False, kernels="plain")
+    again = helpers.replay(plain, steps)
+    _check(again, folder, {"x": toks}, dtype, "long decoding, plain kernels")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_a_kind_are_made_again_from_the_launches_of_the_first(model_dirs, dtype):
+    """Seven layers of one kind (the second mixer, with its convolution's state, and experts): the first makes the
+    rotation's table, the second is recorded, layers after it are its launches with their own tensors, pages and state,
+    the last prepares no next norm and is walked; the same bits as with every layer walked, and the plain
+    implementation's logits."""
+    import tekilix_cases
+    from glassbox_amd import ops
+    from glassbox_amd.engine import Engine
+    layer = copy.deepcopy(CASES["E"]["layers"][1])
+    # (two layers with tensors of their own, used in turn: a layer followed by itself prepares its own first norm, which
+    # is then one tensor in two places of the launches, and such a layer is walked)
+    layers = [layer, copy.deepcopy(layer), dict(layer, weights_of=0), dict(layer, weights_of=1), dict(layer, weights_of=2),
+              dict(layer, weights_of=3), dict(layer, weights_of=0)]
+    tekilix_cases.CASES["taped"] = dict(CASES["E"], layers=layers)
+    try:
+        folder = folder_of(model_dirs.base, "taped")
+    finally:
+        del tekilix_cases.CASES["taped"]
+    requests = {"a": helpers.random_tokens(97, 150, seed=1), "b": helpers.random_tokens(97, 41, seed=2)}
+    steps = helpers.schedule_whole(requests) + helpers.schedule_chunks(requests, (70, 3, 40))
+    before = ops.TAPE_COUNTS["replayed_layers"]
+    taped = helpers.replay(Engine(folder, dtype=dtype, max_tokens=512, max_seqs=2), steps)
+    assert ops.TAPE_COUNTS["replayed_layers"] >= before + 3 * len(steps)
+    before = ops.TAPE_COUNTS["replayed_layers"]
+    walked = helpers.replay(Engine(folder, dtype=dtype, max_tokens=512, max_seqs=2, layer_tapes=False), steps)
+    assert ops.TAPE_COUNTS["replayed_layers"] == before
+    assert all(np.array_equal(taped[r], walked[r]) for r in requests)
+    if dtype == "float32":
+        whole = helpers.replay(Engine(folder, dtype=dtype, max_tokens=512, max_seqs=2), helpers.schedule_whole(requests))
+        _check(whole, folder, requests, dtype, "layers made again")
+
+
+def test_slots_and_pages_that_are_used_again(model_dirs):
+    """Two slots, six requests one after the other in pairs: a request finds the slot (the convolution's last rows) and the
+    pages of one that ended, and must start from nothing."""
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, "D")
+    requests = {r: helpers.random_tokens(160, n, seed=70 + n) for r, n in {"p": 50, "q": 31, "r": 18, "s": 64, "t": 2, "u": 45}.items()}
+    eng = Engine(folder, dtype="float32", max_tokens=128, max_seqs=2)
+    _poison(eng)
+    steps, _ = helpers.schedule_mixed(requests, seed=5, live=2, tail=6)
+    got = helpers.replay(eng, steps)
+    _check(got, folder, requests, "float32", "slots used again")
+
+
+def test_batches_of_unequal_requests_give_each_what_it_gets_alone(model_dirs):
+    """In 32-bit a request's logits do not depend on what else is in its batch, beyond rounding of the sums' order."""
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, "B")
+    requests = _requests(130, seed=4)
+    eng = Engine(folder, dtype="float32", max_tokens=1024, max_seqs=6)
+    alone = helpers.replay(eng, helpers.schedule_whole(requests))
+    together = helpers.replay(eng, [{"entries": [(r, t, list(range(len(t)))) for r, t in requests.items()], "end": list(requests)}])
+    for r in requests:
+        assert np.abs(alone[r] - together[r]).max() < 2e-5 * max(1.0, float(np.abs(alone[r]).max()))
+
+
+# ------------------------------------------------------------------------------------------ generation
+def _greedy(cfg, w, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(torch.argmax(pt.forward(cfg, w, toks)[-1])))
+    return toks[len(prompt):]
+
+
+@pytest.mark.parametrize("name", ["A", "E"])
+def test_greedy_generation_through_the_entry_points(model_dirs, name):
+    from glassbox_amd.engine import Engine, generate, greedy
+    folder = folder_of(model_dirs.base, name, seed=2)
+    cfg, w = pt.load_folder(folder)
+    vocab = CASES[name]["vocab"]
+    prompts = [helpers.random_tokens(vocab, n, seed=50 + n) for n in (5, 44, 1, 23, 70)]
+    want = [_greedy(cfg, w, p, 12) for p in prompts]
+    # (the embedding's table is the head as well, and with random weights a reply mostly settles on one token: which one
+    # depends on the prompt)
+    assert len({tuple(r) for r in want}) > 2, "replies that do not depend on the prompt show nothing"
+    eng = Engine(folder, dtype="float32", max_tokens=1024, max_seqs=3)
+    assert greedy(eng, prompts[1], 12) == want[1]
+    # the scheduler: three live requests at most, prompts in portions of at most 16 tokens beside decoding requests
+    assert generate(eng, prompts, max_tokens=12, token_budget=16, max_seqs=3) == want
+    assert eng.cache.num_seqs() == 0 and eng.cache.free_state_slots() == 3
+
+
+def test_the_command_line_runs_the_model(model_dirs, tmp_path):
+    folder = folder_of(model_dirs.base, "B", seed=2)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    run = lambda *args, stdin=None: subprocess.run([sys.executable, os.path.join(root, "bin", "glassbox"), *args],
+                                                   capture_output=True, text=True, timeout=600, input=stdin)
+    r = run("generate", "--model", folder, "--prompt", "5,17,3,99,41", "-n", "8", "--dtype", "float32", "--no-prefix-cache")
+    assert r.returncode == 0, r.stderr
+    cfg, w = pt.load_folder(folder)
+    assert [int(t) for t in r.stdout.split()] == _greedy(cfg, w, [5, 17, 3, 99, 41], 8)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3, 9], "want": [1, 3]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": [8], "want": [0]}, {"id": "b", "tokens": [4, 4], "want": []}], "end": ["a"]}]
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", str(tmp_path / "o"),
+                        "--max-tokens", "128"], capture_output=True, text=True, timeout=600,
+                       input="".join(json.dumps(s) + "\n" for s in steps))
+    assert r.returncode == 0 and r.stdout.split() == ["done", "0", "done", "1"], r.stderr
+    want = pt.forward(cfg, w, [5, 17, 3, 9, 8]).numpy()
+    assert np.abs(np.fromfile(tmp_path / "o" / "0.f32", dtype="<f4").reshape(2, -1) - want[[1, 3]]).max() < 1e-4
+    assert np.abs(np.fromfile(tmp_path / "o" / "1.f32", dtype="<f4") - want[4]).max() < 1e-4
