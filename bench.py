@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers 24]
                     [--shapes smollm2-1.7b|smollm2-360m|llama-3-8b] [--reps 3]
-    python bench.py --design sagalorn|dekinex|vumalix [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
+    python bench.py --design sagalorn|dekinex|vumalix|tekilix [--design-sizes 360m,1.7b] [--layers 12] [--batch 8] [--context 4096]
 
 ``--design sagalorn`` is another measurement with a line of its own: prefill and decode throughput of Sagalorn models
 whose layers have the sizes of the named shapes (a third of the layers each retention, windowed attention with kept
@@ -21,6 +21,13 @@ size plus half as many rotated columns, a query latent of 3/8 and a key/value la
 1,024) to one of differential attention (two maps of half the head size a head), every mixer behind a convolution of
 the residual over four tokens, every layer with a polynomial feed-forward of one and a half times the Llama's
 intermediate size (two matrices where the Llama has three: the same bytes and multiply-adds).
+
+``--design tekilix`` does the same for Tekilix models: the two gated attention mixers in turn (biased projections, one
+norm over all of q and of k, capped scores and a sink of score 0; and q and k behind a convolution of four taps with the
+keys as values, stretched rotation and learned sinks), both within runs of 1,024 positions, bounded norms around every
+sublayer, and in every layer routed experts of squared-ReLU units (eight in four groups of which two are kept, two a
+token, each 3/8 of the Llama's intermediate size, and a shared one of 3/4: as many multiply-adds a token as the Llama's
+three matrices).
 
 A step is one decode step of the whole batch through the path that greedy generation uses: ``Engine.step``
 (which replays steps of single tokens from HIP graphs) and the device sampler (``sampling.greedy_pending``), the
@@ -112,7 +119,26 @@ def vumalix_like(shapes: dict, layers: int, window: int = 1024) -> dict:
                 layers=[kinds[i % 3] for i in range(layers)])
 
 
-DESIGNS = {"sagalorn": ("Sagalorn", sagalorn_like), "dekinex": ("Dekinex", dekinex_like), "vumalix": ("Vumalix", vumalix_like)}
+def tekilix_like(shapes: dict, layers: int, run: int = 1024, experts: int = 8, top: int = 2) -> dict:
+    """A Tekilix configuration with the widths of a Llama one: the two mixers in turn, routed experts in every layer with
+    as many multiply-adds a token as the Llama's feed-forward."""
+    d, H, G = shapes["hidden_size"], shapes["num_attention_heads"], shapes["num_key_value_heads"]
+    hd = shapes.get("head_dim") or d // H
+    ff = shapes["intermediate_size"]
+    moe = {"kind": "moe", "expert": {"ff": ff * 3 // 8 // 8 * 8}, "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}},
+           "shared": {"ff": ff * 3 // 4 // 8 * 8}}
+    one = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
+           "rot": {"dims": hd // 2, "base": 10000.0}, "mask": {"size": run}}
+    two = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "conv": 4,
+           "rot": {"dims": hd // 2, "base": 250000.0, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}},
+           "mask": {"size": run}}
+    kinds = [{"type": "attention", "mixer": one, "mlp": moe}, {"type": "attention_2", "mixer": two, "mlp": moe}]
+    return dict(architecture="Tekilix", vocab=shapes["vocab_size"], width=d, norm={"eps": shapes["rms_norm_eps"]},
+                embedding={"scale": 1.0}, logit_scale=1.0, layers=[kinds[i % 2] for i in range(layers)])
+
+
+DESIGNS = {"sagalorn": ("Sagalorn", sagalorn_like), "dekinex": ("Dekinex", dekinex_like), "vumalix": ("Vumalix", vumalix_like),
+           "tekilix": ("Tekilix", tekilix_like)}
 
 
 def design_bench(a) -> int:

@@ -197,6 +197,40 @@ __global__ void relu2_units_kernel(const I* __restrict__ z, int ld, const float*
   act[(size_t)t * lda + j] = from_f<O>(y);
 }
 
+// The same, eight columns a thread (rows of whole 16-byte words, experts of whole groups of eight columns).
+template <typename I>
+__global__ void relu2_units_words_kernel(const I* __restrict__ z, int ld, const float* __restrict__ combine, int cols, bf16* __restrict__ act,
+                                         int lda, long long count, int inter, int E, int ff) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= count) return;
+  const int words = inter / 8;
+  const long long t = idx / words;
+  const int j = (int)(idx % words) * 8;
+  const float w = combine ? combine[(size_t)t * cols + (j < E * ff ? j / ff : E)] : 1.f;
+  bf16x8 o;
+  if (w != 0.f) {
+    float v[8];
+    if constexpr (std::is_same<I, float>::value) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(z + (size_t)t * ld + j), b = *reinterpret_cast<const f32x4*>(z + (size_t)t * ld + j + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = a[e], v[4 + e] = b[e];
+    } else {
+      const bf16x8 a = *reinterpret_cast<const bf16x8*>(z + (size_t)t * ld + j);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (float)a[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float r = fmaxf(v[e], 0.f);
+      o[e] = (bf16)(r * r * w);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)0.f;
+  }
+  *reinterpret_cast<bf16x8*>(act + (size_t)t * lda + j) = o;
+}
+
 // counts[e]: how many of the n * top entries chose expert e.  One workgroup an expert.
 __global__ __launch_bounds__(256) void count_kernel(const int32_t* __restrict__ ids, int entries, int32_t* __restrict__ counts) {
   __shared__ int part[4];
@@ -336,6 +370,14 @@ extern "C" int gb_moe_relu2_units(const void* z, int in_dtype, int ld, const flo
   if (n == 0) return 0;
   const long long count = (long long)n * inter;
   GB_REQUIRE((count + 255) / 256 < (1ll << 31), "moe_relu2_units: too many elements");
+  if (out_dtype == kBF16 && inter % 8 == 0 && ff % 8 == 0 && ld % 8 == 0 && lda % 8 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)act % 16 == 0) {
+    const dim3 wgrid((unsigned)((count / 8 + 255) / 256));
+    if (in_dtype == kF32)
+      hipLaunchKernelGGL(relu2_units_words_kernel<float>, wgrid, dim3(256), 0, stream, (const float*)z, ld, combine, cols, (bf16*)act, lda, count / 8, inter, E, ff);
+    else
+      hipLaunchKernelGGL(relu2_units_words_kernel<bf16>, wgrid, dim3(256), 0, stream, (const bf16*)z, ld, combine, cols, (bf16*)act, lda, count / 8, inter, E, ff);
+    return launched("moe_relu2_units");
+  }
   const dim3 grid((unsigned)((count + 255) / 256));
   if (in_dtype == kF32 && out_dtype == kF32)
     hipLaunchKernelGGL((relu2_units_kernel<float, float>), grid, dim3(256), 0, stream, (const float*)z, ld, combine, cols, (float*)act, lda, count, inter, E, ff);

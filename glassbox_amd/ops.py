@@ -94,9 +94,9 @@ _SIGS = {
         "gb_tanh_norm": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
         # x, y, slices, slice stride, alpha, w, b, next alpha, w, b, h, its dtype, n, d, stream
         "gb_tanh_norm_add": [_vp, _vp, _i, C.c_longlong, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
-        # proj, dtype, ld, bias, wconv, taps, state, tok_seq, q_start, pos0, state slots, flags, wq, wk, eps, cos, sin,
+        # proj, dtype, ld, bias, wconv, sums, state, tok_seq, q_start, pos0, state slots, flags and taps, wq, wk, eps, cos, sin,
         # rot, mag, out, ldo, hd, slots, k, v, page, n, H, G, dk, dv, stream
-        "gb_qk_heads": [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _f, _vp, _i,
+        "gb_qk_heads": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _i, _f, _vp, _i,
                         _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
         # proj, dtype, ld, bias, state, q_start, q_len, state slots, requests, channels, taps, stream
         "gb_qk_conv_state": [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
@@ -1504,7 +1504,6 @@ def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: 
 
 
 ROPE_PRODUCT_MAX_ROWS = 64
-QK_HEADS_MAX_CHANNELS = 15872   # tanhmix.hip stages a token's query and key channels in 64 KB of LDS
 
 
 def gemm_rope(a: torch.Tensor, w: torch.Tensor, qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int,
@@ -1821,7 +1820,7 @@ def qk_heads(proj: torch.Tensor, ctx, out: torch.Tensor, head_cols: int, n_heads
     """The query, key and value heads of every row of the step as attention reads them, ``out`` [n, (heads + 2 kv heads) *
     head_cols], from the stacked projections ``proj`` ([n, query channels | key channels | value channels | ...]; with
     ``tied`` there are no value channels: the key channels, biased and convolved, are the values):
-    ``bias`` (float32, one a channel) is added; ``wconv`` ([query + key channels, taps] float32) convolves every query and
+    ``bias`` (float32, one a channel) is added; ``wconv`` ([taps, query + key channels] float32, a row a tap) convolves every query and
     key channel over the request's earlier rows and its ``state`` slot ([slots, taps - 1, channels] float32, moved on here
     in a step of single tokens, else by ``qk_conv_state``); an RMS norm over all query (key) channels at once with a weight a
     channel (``joint``) or over each head with ``dim`` weights that the heads share; the first ``rot`` channels of each
@@ -1832,8 +1831,8 @@ def qk_heads(proj: torch.Tensor, ctx, out: torch.Tensor, head_cols: int, n_heads
     channels = (n_heads + n_kv_heads) * dim
     taps = 0
     if wconv is not None:
-        taps = wconv.shape[1]
-        _f32_rows(wconv, (channels, taps), "qk_heads: wconv")
+        taps = wconv.shape[0]
+        _f32_rows(wconv, (taps, channels), "qk_heads: wconv")
         if taps > 1 and (state is None or state.dtype != torch.float32 or not state.is_contiguous()
                          or tuple(state.shape[1:]) != (taps - 1, channels)):
             raise KernelError(f"qk_heads: state must be contiguous float32 [slots, {taps - 1}, {channels}]")
@@ -1852,10 +1851,13 @@ def qk_heads(proj: torch.Tensor, ctx, out: torch.Tensor, head_cols: int, n_heads
         if nkv != n_kv_heads or hd != head_cols:
             raise KernelError("qk_heads: the pages hold other heads than these")
     single = 1 if ctx.host["n_decode"] == ctx.num_seqs else 0
+    # one norm over a whole row: the rows' squares are added up in a pass of their own, which every (token, head) then reads
+    sums = ctx.buffer("qk_heads_sums", (n, 2), torch.float32) if joint else None
     lib = _lib("tanhmix")
-    _launch(lib, lib.gb_qk_heads, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(bias), _p(wconv), int(taps), _p(state),
+    _launch(lib, lib.gb_qk_heads, _p(proj), dtype_code(proj), _rows(proj, "proj"), _p(bias), _p(wconv), _p(sums), _p(state),
             _p(ctx.tok_seq), _p(ctx.q_start), _p(ctx.pos0), _p(ctx.state_slots),
-            single | (2 if joint else 0) | (4 if neighbours else 0) | (8 if tied else 0), _p(norm_q), _p(norm_k), float(eps),
+            single | (2 if joint else 0) | (4 if neighbours else 0) | (8 if tied else 0) | (int(taps) << 8), _p(norm_q), _p(norm_k),
+            float(eps),
             _p(cos), _p(sin), int(rot), float(magnitude), _p(out), _rows(out, "out"), int(head_cols), _p(slots), _p(k_pages),
             _p(v_pages), int(page), n, n_heads, n_kv_heads, dim, vdim, _stream())
     if taps > 1 and not single:

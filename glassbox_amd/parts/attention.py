@@ -564,6 +564,8 @@ class GatedAttention(Mixer):
             raise ValueError(f"{rot_dims} rotated channels: an even number up to the key size {dim}")
         if tied_values and vdim != dim:
             raise ValueError(f"values that are the keys have the keys' size: dim {dim}, vdim {vdim}")
+        if qk_norm == "joint" and taps:
+            raise ValueError("one norm over all of q (and of k) behind a convolution is not served: qk_norm='head' goes with taps")
         if qk_norm not in ("joint", "head") or rot_pairs not in ("neighbours", "halves") or sink not in (None, "zero", "learned") \
                 or gate not in ("head", "channel"):
             raise ValueError("qk_norm: joint | head; rot_pairs: neighbours | halves; sink: None | zero | learned; gate: head | channel")
@@ -610,7 +612,8 @@ class GatedAttention(Mixer):
             self.b_in = torch.cat([tensors["q.b"], tensors["k.b"]] + ([] if self.tied_values else [tensors["v.b"]])).float().contiguous()
         self.norm_q, self.norm_k = tensors["q.norm"].float().contiguous(), tensors["k.norm"].float().contiguous()
         if self.taps:
-            self.wconv = torch.cat([tensors["q.conv"], tensors["k.conv"]], 0).float().contiguous()
+            # a row a tap: neighbouring channels' weights of one tap lie side by side
+            self.wconv = torch.cat([tensors["q.conv"], tensors["k.conv"]], 0).float().t().contiguous()
         if self.sink == "learned":
             self.sinks = tensors["sink"].float().contiguous()
         elif self.sink == "zero":
@@ -626,9 +629,6 @@ class GatedAttention(Mixer):
                                f"the attention kernels take"))
         if self.taps > ops.CONV_MAX_TAPS:
             out.append(("taps", f"{self.taps} is above {ops.CONV_MAX_TAPS}, the longest convolution the kernel takes"))
-        if self.channels > ops.QK_HEADS_MAX_CHANNELS:
-            out.append(("dim", f"{self.channels} query and key channels a token are above {ops.QK_HEADS_MAX_CHANNELS}, the most "
-                               f"the kernel that prepares the heads stages"))
         return out
 
     def forward(self, ctx, h, residual, cache: Optional[LayerCache], store: bool = False):

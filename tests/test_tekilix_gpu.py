@@ -36,9 +36,11 @@ def _step_ctx(rows, slots):
     lens = [b - a for _, a, b in rows]
     starts = np.cumsum([0] + lens)[:-1]
     tok_seq = [s for s, n in enumerate(lens) for _ in range(n)]
+    from glassbox_amd.engine.context import Workspace
     return SimpleNamespace(q_start=_i32(starts), q_len=_i32(lens), pos0=_i32(a for _, a, _ in rows), tok_seq=_i32(tok_seq),
                            state_slots=_i32(slots[r] for r, _, _ in rows), num_seqs=len(rows),
-                           host={"max_q_len": max(lens), "n_decode": sum(1 for n in lens if n == 1)})
+                           host={"max_q_len": max(lens), "n_decode": sum(1 for n in lens if n == 1)},
+                           buffer=Workspace(torch.device(DEV)).buffer)
 
 
 def _pool(T, P, G, hc, dtype, seed=0):
@@ -167,7 +169,7 @@ def test_heads_prepared_in_portions_of_a_batch(kind, m, dtype):
     channels = (H + G) * dk
     state = torch.full((5, taps - 1, channels), 55.0, device=DEV) if taps > 1 else None
     bias = _dev(torch.cat([w["x.q.b"], w["x.k.b"], w["x.v.b"]])) if kind == "attention" else None
-    wconv = _dev(torch.cat([w["x.q.conv"], w["x.k.conv"]], 0)) if taps else None
+    wconv = _dev(torch.cat([w["x.q.conv"], w["x.k.conv"]], 0).t()) if taps else None   # a row a tap
     rot = m.get("rot")
     rotary = Rotary(rot["dims"], rot["base"], tuple(rot["scaling"][k] for k in ("factor", "original", "fast", "slow"))
                     if rot.get("scaling") else None) if rot else None
