@@ -735,6 +735,20 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
     load_keys<HD, T>(kf, src, kb, lane);
     load_values<HD, T>(vf, src, kb, lane);
     if (has_second) {
+      // the tiles in order: the kept first keys (both blocks); the earlier block's tiles that lie before everything
+      // the later block sees (its window, or its run of positions, begins behind them: the earlier block alone); the
+      // tiles both see; then the later block alone
+      const int kept_tiles = (keep + 63) & ~63;
+      while (kb <= range[0].last && kb < kept_tiles) {
+        const int next = my_next(kb);
+        attend64_q32<HD, 2, 3, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, true, c, lane, keep, cap_in, cap_out);
+        kb = next;
+      }
+      while (kb <= range[0].last && kb + 63 < range[1].first) {
+        const int next = my_next(kb);
+        attend64_q32<HD, 2, 1, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep, cap_in, cap_out);
+        kb = next;
+      }
       while (kb <= range[0].last) {
         const int next = my_next(kb);
         const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));

@@ -396,9 +396,26 @@ __global__ __launch_bounds__(256) void row_squares_kernel(const T* __restrict__ 
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * ld;
   float sq = 0.f, sk = 0.f;
-  for (int c = threadIdx.x; c < qd + kd; c += 256) {
-    const float v = to_f(row[c]) + (bias ? bias[c] : 0.f);
-    if (c < qd) sq = fmaf(v, v, sq); else sk = fmaf(v, v, sk);
+  if (std::is_same<T, bf16>::value && qd % 8 == 0 && kd % 8 == 0 && ld % 8 == 0 && (uintptr_t)proj % 16 == 0 && (uintptr_t)bias % 16 == 0) {
+    for (int c = threadIdx.x * 8; c < qd + kd; c += 256 * 8) {   // a word of eight channels a thread
+      const bf16x8 x = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const bf16*>(row) + c);
+      float b[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) b[e] = 0.f;
+      if (bias) load8f(bias + c, b);
+      float part = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float v = (float)x[e] + b[e];
+        part = fmaf(v, v, part);
+      }
+      if (c < qd) sq += part; else sk += part;
+    }
+  } else {
+    for (int c = threadIdx.x; c < qd + kd; c += 256) {
+      const float v = to_f(row[c]) + (bias ? bias[c] : 0.f);
+      if (c < qd) sq = fmaf(v, v, sq); else sk = fmaf(v, v, sk);
+    }
   }
   sq = block_sum(sq, scratch);
   sk = block_sum(sk, scratch);
