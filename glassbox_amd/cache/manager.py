@@ -11,7 +11,7 @@ from typing import List, Optional, Sequence, Tuple
 
 from .. import build
 
-FULL, WINDOW = 0, 1
+FULL, WINDOW, RUNS = 0, 1, 2
 
 
 class OutOfPages(RuntimeError):
@@ -25,7 +25,8 @@ class CacheError(RuntimeError):
 @dataclass(frozen=True)
 class GroupSpec:
     """One pool of pages: ``kind`` FULL keeps every key, WINDOW only the last ``window`` and, with ``keep_first``, the
-    first so many for as long as the request lives.  (The order of the fields is that of earlier callers.)"""
+    first so many for as long as the request lives; RUNS the keys of the run of ``window`` positions (runs counted from
+    position 0) that holds the next query.  (The order of the fields is that of earlier callers.)"""
     kind: int = FULL
     window: int = 0
     num_pages: int = 0
@@ -88,8 +89,8 @@ class CacheManager:
         if page_size <= 0:
             raise CacheError("page_size must be positive")
         for g in groups:
-            if g.kind == WINDOW and g.window <= 0:
-                raise CacheError("a window group needs a positive window")
+            if g.kind in (WINDOW, RUNS) and g.window <= 0:
+                raise CacheError("a window group needs a positive window, a group of runs a positive run")
             if g.keep_first < 0 or (g.keep_first and g.kind != WINDOW):
                 raise CacheError("kept first keys go with a window group")
             if g.num_pages <= 0:

@@ -188,8 +188,9 @@ int CacheManager::commit(int64_t id, const int32_t* tokens, int n) {
   // pages that every later query's window has passed go back to their pool
   for (size_t gi = 0; gi < groups_.size(); ++gi) {
     Group& g = groups_[gi];
-    if (g.spec.kind != kWindow) continue;
-    int first_needed = s.len - g.spec.window + 1;  // oldest key the next query reads
+    if (g.spec.kind != kWindow && g.spec.kind != kRuns) continue;
+    // oldest key the next query reads: the window's first, or the first of the run that holds position len
+    int first_needed = g.spec.kind == kRuns ? s.len - s.len % g.spec.window : s.len - g.spec.window + 1;
     if (first_needed <= 0) continue;
     int dead = first_needed / page_size_;          // pages [0, dead) lie wholly before it
     int kept = (g.spec.keep_first + page_size_ - 1) / page_size_;   // pages that hold a key every query reads
@@ -211,10 +212,10 @@ int CacheManager::truncate(int64_t id, int len) {
   if (len > s.len || len < 0) return -2;
   for (size_t gi = 0; gi < groups_.size(); ++gi) {
     const Group& g = groups_[gi];
-    if (g.spec.kind != kWindow) continue;
-    int first_needed = std::max(0, len - g.spec.window + 1);
+    if (g.spec.kind != kWindow && g.spec.kind != kRuns) continue;
+    int first_needed = g.spec.kind == kRuns ? len - len % g.spec.window : std::max(0, len - g.spec.window + 1);
     for (int j = first_needed / page_size_; j < (len + page_size_ - 1) / page_size_; ++j)
-      if (s.tables[gi][j] < 0) return -3;  // the window would reach into pages already given back
+      if (s.tables[gi][j] < 0) return -3;  // the window (or the run) would reach into pages already given back
   }
   s.len = len;
   if ((int)s.tokens.size() > len) s.tokens.resize(len);

@@ -17,11 +17,13 @@
 
 namespace gb {
 
-enum GroupKind : int { kFull = 0, kWindow = 1 };
+enum GroupKind : int { kFull = 0, kWindow = 1, kRuns = 2 };
 
 struct GroupSpec {
   int kind = kFull;
   int window = 0;      // kWindow: a query at position p reads keys p-window+1 .. p
+                       // kRuns: positions are cut into runs of `window` from 0 on, and a query reads the keys of its own
+                       // run up to itself: the pages that lie wholly before the next query's run are given back
   int keep_first = 0;  // kWindow: and keys 0 .. keep_first-1, whose pages are never given back while the request lives
   int num_pages = 0;
 };

@@ -12,7 +12,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import torch
 
 from .. import ops
-from ..cache.manager import FULL, CacheManager, GroupSpec, OutOfPages
+from ..cache.manager import FULL, RUNS, CacheManager, GroupSpec, OutOfPages
 from ..parts.base import LayerCache
 from ..sampling.pending import PendingToken, entry_values, place_pending
 from ..config import config_from_dir
@@ -50,9 +50,12 @@ def sharing_obstacles(model) -> List[str]:
     can).  Sharing hands a new request the pages that another wrote and skips those tokens, in every layer at once,
     so every cache layer must still hold them and must need nothing else to go on from there."""
     windows: Dict[int, List[int]] = {}
+    runs: Dict[int, List[int]] = {}
     stateful: List[int] = []
     for c, (spec, state) in enumerate(zip(model.cache_specs(), model.state_specs())):
-        if spec is not None and spec.kind != FULL:
+        if spec is not None and spec.kind == RUNS:
+            runs.setdefault(spec.window, []).append(c)
+        elif spec is not None and spec.kind != FULL:
             windows.setdefault(spec.window, []).append(c)
         if state is not None:
             stateful.append(c)
@@ -61,6 +64,9 @@ def sharing_obstacles(model) -> List[str]:
     for window, cs in sorted(windows.items()):
         lines.append(f"{several(cs)}: a window of {window} positions, whose pages are given back as soon as the window "
                      f"has passed them, so that a later request does not find them")
+    for run, cs in sorted(runs.items()):
+        lines.append(f"{several(cs)}: runs of {run} positions, whose pages are given back as soon as a run has ended, so "
+                     f"that a later request does not find them")
     if stateful:
         lines.append(f"{several(stateful)}: state of its own for each request, which a request that skips tokens would "
                      f"need as it was at the edge of the last shared page")

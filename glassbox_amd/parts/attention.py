@@ -15,7 +15,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from .base import (FULL, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, StateSpec, TensorSpec, emit_target,
+from .base import (FULL, RUNS, WINDOW, CacheSpec, LayerCache, Mixer, PositionEncoding, PreNormed, StateSpec, TensorSpec, emit_target,
                    needs_multiple_of_8, product, product_in_slices, split_workspace)
 
 
@@ -578,7 +578,8 @@ class GatedAttention(Mixer):
         self.value_cols = 0 if tied_values else n_kv_heads * vdim
         self.gate_cols = n_heads if gate == "head" else n_heads * vdim
         self.position = Rotary(rot_dims, rot_base, rot_scaling) if rot_dims else None
-        self.cache_spec = CacheSpec(n_kv_heads, self.head_cols, FULL, 0)
+        # (the pages of a run that has ended are given back: no later token reads them)
+        self.cache_spec = CacheSpec(n_kv_heads, self.head_cols, RUNS if self.chunk else FULL, self.chunk)
         self.state_spec = StateSpec((self.taps - 1, self.channels), torch.float32, 0.0) if self.taps > 1 else None
         self.w_in = self.wo = self.b_in = self.wconv = self.norm_q = self.norm_k = self.sinks = None
 

@@ -40,7 +40,7 @@ from typing import Dict, Iterator, List, NamedTuple, Optional, Tuple
 
 import torch
 
-FULL, WINDOW = 0, 1
+FULL, WINDOW, RUNS = 0, 1, 2
 
 
 @dataclass(frozen=True)
@@ -58,7 +58,8 @@ class TensorSpec:
 @dataclass(frozen=True)
 class CacheSpec:
     """Paged keys and values of one layer.  kind FULL keeps every position, WINDOW the last ``window`` and, with
-    ``keep_first``, the first so many as well."""
+    ``keep_first``, the first so many as well; RUNS the positions of the run of ``window`` (runs counted from the
+    request's first position) that holds the next query."""
     num_kv_heads: int
     head_dim: int
     kind: int = FULL
@@ -68,7 +69,7 @@ class CacheSpec:
     @property
     def group_key(self) -> Tuple[int, int, int]:
         windowed = self.kind == WINDOW
-        return (self.kind, self.window if windowed else 0, self.keep_first if windowed else 0)
+        return (self.kind, self.window if self.kind != FULL else 0, self.keep_first if windowed else 0)
 
 
 @dataclass(frozen=True)

@@ -192,6 +192,35 @@ def test_window_group_gives_pages_back_as_the_window_passes():
     assert kv.used_pages(0) == 0 and kv.used_pages(1) == 0
 
 
+def test_a_group_of_runs_gives_pages_back_when_a_run_has_ended():
+    from glassbox_amd.cache.manager import RUNS
+    kv = CacheManager(16, [GroupSpec(FULL, 0, 16), GroupSpec(RUNS, 40, 16)], 0, True)
+    assert not kv.share_prefixes        # a page of a run that has ended cannot be offered to others
+    kv.add_seq(7, [])
+    toks = list(range(130))
+    kv.reserve(7, 39); kv.commit(7, toks[:39])
+    assert all(p >= 0 for p in kv.table(7, 1))      # the next query, position 39, still reads its run from 0 on
+    kv.reserve(7, 1); kv.commit(7, toks[39:40])
+    # the next query is position 40, the first of its run: pages 0 and 1 (0..31) are dead, page 2 (32..47) holds 40..47
+    assert [p >= 0 for p in kv.table(7, 1)] == [False, False, True]
+    for i in range(40, 130):
+        kv.reserve(7, 1); kv.commit(7, [toks[i]])
+        kv.check_invariants()
+        first_needed = (i + 1) - (i + 1) % 40
+        table = kv.table(7, 1)
+        assert all((p == -1) == ((j + 1) * 16 <= first_needed) for j, p in enumerate(table)), (i, table)
+        assert kv.used_pages(1) <= 4
+    assert kv.used_pages(0) == 9
+    with pytest.raises(CacheError, match="given back"):
+        kv.truncate(7, 119)              # position 119 would read 80..119, and 80..95 went back at length 120
+    kv.truncate(7, 125)
+    kv.remove_seq(7)
+    kv.check_invariants()
+    assert kv.used_pages(0) == 0 and kv.used_pages(1) == 0
+    with pytest.raises(CacheError):
+        CacheManager(16, [GroupSpec(RUNS, 0, 16)], 0, False)
+
+
 def test_a_portion_larger_than_the_window_needs_its_pages_for_one_step():
     kv = CacheManager(16, [GroupSpec(WINDOW, 8, 4)], 0, False)
     kv.add_seq(1, [])

@@ -239,6 +239,8 @@ def test_the_model_declares_the_checkpoints_tensors_and_one_cache_layer_a_call(f
             spec, state = model.cache_specs()[call.cache], model.state_specs()[call.cache]
             m = layer["mixer"]
             assert spec.num_kv_heads == m["kv_heads"] and spec.head_dim >= max(m["dim"], m["vdim"])
+            run = (m.get("mask") or {"size": 0})["size"]      # a layer that sees runs keeps the pages of the run at hand
+            assert (spec.kind, spec.window) == ((2, run) if run else (0, 0))
             taps = m.get("conv", 0) if layer["type"] == "attention_2" else 0
             assert (state is None) == (taps <= 1)
             if state is not None:

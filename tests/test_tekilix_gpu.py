@@ -611,6 +611,22 @@ def test_layers_of_a_kind_are_made_again_from_the_launches_of_the_first(model_di
         _check(whole, folder, requests, dtype, "layers made again")
 
 
+def test_a_pool_that_holds_runs_not_requests(model_dirs):
+    """A request of 600 tokens in a pool of 256: every layer of the model sees runs of positions, and the pages of a run
+    that has ended go back to the pool while the request lives (portions of 100, then single tokens)."""
+    from glassbox_amd.engine import Engine
+    folder = folder_of(model_dirs.base, "E")      # runs of 16 and 40 positions
+    toks = helpers.random_tokens(97, 600, seed=31)
+    eng = Engine(folder, dtype="float32", max_tokens=256, max_seqs=2)
+    _poison(eng)
+    steps = helpers.schedule_chunks({"x": toks[:520]}, (100,))
+    steps[-1]["end"] = []
+    steps += [{"entries": [("x", [t], [0])], "end": ["x"] if i == 79 else []} for i, t in enumerate(toks[520:])]
+    got = helpers.replay(eng, steps)
+    _check(got, folder, {"x": toks}, "float32", "a pool smaller than its request")
+    assert all(eng.cache.used_pages(g) == 0 for g in range(len(eng.group_keys)))
+
+
 def test_slots_and_pages_that_are_used_again(model_dirs):
     """Two slots, six requests one after the other in pairs: a request finds the slot (the convolution's last rows) and the
     pages of one that ended, and must start from nothing."""
