@@ -58,8 +58,12 @@ __device__ __forceinline__ int first_key(int pos, int window, int span) {
   return span > 0 ? pos - pos % span : window > 0 ? max(0, pos - window + 1) : 0;
 }
 
-// tanh by one exponential: 1 - 2 / (1 + e^(2x)); +-1 where the exponential leaves the range
-__device__ __forceinline__ float tanh_fast(float x) { return 1.0f - 2.0f * __frcp_rn(1.0f + __expf(2.0f * x)); }
+// out * tanh(x * in) by one exponential and one reciprocal (the hardware's approximations, an ulp each):
+// out - 2 out / (1 + 2^(x * in * 2 log2(e))); +-out where the exponential leaves the range
+__device__ __forceinline__ float capped_fast(float x, float in, float out) {
+  const float e = __builtin_amdgcn_exp2f(x * (in * 2.8853900817779268f));
+  return fmaf(-2.0f * out, __builtin_amdgcn_rcpf(1.0f + e), out);
+}
 
 template <int HD>
 struct Running {
@@ -83,7 +87,7 @@ __device__ __forceinline__ void reset(Running<HD>& st) {
 // their keys are masked anyway.
 // WIDE: the softmax weights enter the value product in two bfloat16 parts, p = hi + lo (two products), which keeps 16
 // bits of them instead of 8: for results that go on in 32-bit.
-template <int HD, bool WIDE = false>
+template <int HD, bool WIDE = false, bool CAP = false>
 __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, const bf16* __restrict__ kp,
                                          const bf16* __restrict__ vp, const int32_t* __restrict__ table, int nkv, int kvh,
                                          int P, int kbase, int lo, int hi, int clamp_lo, int clamp_hi, float scale,
@@ -121,7 +125,7 @@ __device__ __forceinline__ void attend64(Running<HD>& st, const bf16x8* qf, cons
     for (int r = 0; r < 4; ++r) {
       const int key = kbase + 16 * t + 4 * c + r;
       float sc = a[r] * scale;
-      if (softcap > 0.f) sc = softcap * tanh_fast(sc / softcap);   // (the same for the whole wave)
+      if (CAP) sc = capped_fast(a[r], scale / softcap, softcap);   // (a kernel of its own: the others' score loops stay as they were)
       s[t][r] = (key >= lo && key <= hi) ? sc : -INFINITY;
       mx = fmaxf(mx, s[t][r]);
     }
@@ -186,7 +190,7 @@ __device__ __forceinline__ void store_out4(float* p, const f32x4& v) { *reinterp
 // grid (chunks, kv heads, requests); request s is row s of q and out, at position positions[s].
 // WAVES waves take 64 keys each in turn; dynamic LDS holds their partial results for the merge:
 // WAVES * (32 + HD * G) floats, G the query heads per kv head.
-template <int HD, int WAVES, typename OT>
+template <int HD, int WAVES, typename OT, bool CAP = false>
 __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restrict__ q, int q_stride, OT* __restrict__ out,
                                                             int out_stride, float* __restrict__ ws_acc,
                                                             float* __restrict__ ws_ml, const int32_t* __restrict__ positions,
@@ -223,9 +227,9 @@ __global__ __launch_bounds__(WAVES * 64) void decode_kernel(const bf16* __restri
   const int end = min(c0 + chunk, pos + 1);
   for (int kb = c0 + wave * 64; kb < end; kb += 64 * WAVES) {
     // the kept first keys of these 64, then those inside the window (a tile can hold both kinds)
-    if (kb < kept) attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane, ex.softcap);
+    if (kb < kept) attend64<HD, WIDE, CAP>(st, qf, kp, vp, table, nkv, kvh, P, kb, col < G ? 0 : 1, col < G ? kept - 1 : 0, 0, kept - 1, scale, lane, ex.softcap);
     if (kb + 64 <= lo) continue;
-    attend64<HD, WIDE>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane, ex.softcap);
+    attend64<HD, WIDE, CAP>(st, qf, kp, vp, table, nkv, kvh, P, kb, col_lo, col_hi, lo, pos, scale, lane, ex.softcap);
   }
   st.l += __shfl_xor(st.l, 16, kWave);
   st.l += __shfl_xor(st.l, 32, kWave);
@@ -417,7 +421,7 @@ __device__ __forceinline__ void load_values(bf16x8 (&vf)[(HD + 31) / 32][2 * T],
 // registers at a time; as soon as the last block's score products have read kf it is loaded again
 // for the keys from `next`, and vf likewise after the last value products, so that those loads are
 // in flight during the arithmetic in between.
-template <int HD, int QB, int ACT, int T = 2, bool WIDE = false>
+template <int HD, int QB, int ACT, int T = 2, bool WIDE = false, bool CAP = false>
 __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32x16 (&acc)[QB][(HD + 31) / 32],
                                              const bf16x8* __restrict__ q_lds, int q_at, bf16x8 (&kf)[T][HD / 16],
                                              bf16x8 (&vf)[(HD + 31) / 32][2 * T], const PageSource& src, int kbase, int next,
@@ -447,11 +451,11 @@ __device__ __forceinline__ void attend64_q32(float (&m)[QB], float (&l)[QB], f32
       __builtin_amdgcn_sched_barrier(0);
       load_keys<HD, T>(kf, src, next, lane);
     }
-    if (cap_in > 0.f) {  // capped scores, kept in the raw scores' unit (the same for the whole wave)
+    if (CAP) {  // capped scores, kept in the raw scores' unit (a kernel of its own: the others stay as they were)
 #pragma unroll
       for (int t = 0; t < T; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[t][r] = cap_out * tanh_fast(s[t][r] * cap_in);
+        for (int r = 0; r < 16; ++r) s[t][r] = capped_fast(s[t][r], cap_in, cap_out);
     }
     if (mask) {  // the same for the whole wave
 #pragma unroll
@@ -632,7 +636,7 @@ __device__ __forceinline__ void hand_over(float& m, float& l, f32x16 (&acc)[DB],
 // blocks w and n-1-w of 32 tokens.  SPLIT waves share a pair: they take its tiles of 64 keys in turn, and at the
 // end the others hand their sums to the first through LDS.  One wave a pair is best when the pairs alone give
 // every SIMD a wave; short portions and few heads do not, and then the keys are what is left to divide.
-template <int HD, int QB, int PAIRS, int SPLIT, typename OT>
+template <int HD, int QB, int PAIRS, int SPLIT, typename OT, bool CAP = false>
 __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf16* __restrict__ q, int q_stride, OT* __restrict__ out,
                                                       int out_stride, const int32_t* __restrict__ q_start,
                                                       const int32_t* __restrict__ q_len, const int32_t* __restrict__ pos0,
@@ -741,29 +745,29 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       const int kept_tiles = (keep + 63) & ~63;
       while (kb <= range[0].last && kb < kept_tiles) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 3, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, true, c, lane, keep, cap_in, cap_out);
+        attend64_q32<HD, 2, 3, 2, WIDE, CAP>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, true, c, lane, keep, cap_in, cap_out);
         kb = next;
       }
       while (kb <= range[0].last && kb + 63 < range[1].first) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 1, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep, cap_in, cap_out);
+        attend64_q32<HD, 2, 1, 2, WIDE, CAP>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep, cap_in, cap_out);
         kb = next;
       }
       while (kb <= range[0].last) {
         const int next = my_next(kb);
         const bool mask = !(range[0].unmasked(kb) && range[1].unmasked(kb));
-        attend64_q32<HD, 2, 3, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep, cap_in, cap_out);
+        attend64_q32<HD, 2, 3, 2, WIDE, CAP>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, mask, c, lane, keep, cap_in, cap_out);
         kb = next;
       }
       while (kb <= range[1].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 2, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep, cap_in, cap_out);
+        attend64_q32<HD, 2, 2, 2, WIDE, CAP>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[1].unmasked(kb), c, lane, keep, cap_in, cap_out);
         kb = next;
       }
     } else {
       while (kb <= range[0].last) {
         const int next = my_next(kb);
-        attend64_q32<HD, 2, 1, 2, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep, cap_in, cap_out);
+        attend64_q32<HD, 2, 1, 2, WIDE, CAP>(m, l, acc, q_lds, q_at, kf, vf, src, kb, next, lo, hi, !range[0].unmasked(kb), c, lane, keep, cap_in, cap_out);
         kb = next;
       }
     }
@@ -812,7 +816,7 @@ __global__ __launch_bounds__(64 * PAIRS * SPLIT, 2) void prefill_kernel(const bf
       load_keys<HD, T>(kf, src, key_of(i0), lane);
       load_values<HD, T>(vf, src, key_of(i0), lane);
       for (int i = i0; key_of(i) <= range.last; i += stride)
-        attend64_q32<HD, 1, 1, T, WIDE>(m, l, acc, q_lds, q_at, kf, vf, src, key_of(i), key_of(i + stride), lo, hi,
+        attend64_q32<HD, 1, 1, T, WIDE, CAP>(m, l, acc, q_lds, q_at, kf, vf, src, key_of(i), key_of(i + stride), lo, hi,
                                   !range.unmasked(key_of(i), SPAN), c, lane, keep, cap_in, cap_out);
       if constexpr (SPLIT > 1) {
         hand_over<DB, SPLIT>(m[0], l[0], acc[0], handed[wave], handed_ml[wave], half, lane, c, which > 0);
@@ -864,19 +868,30 @@ static int decode_launch(const void* q, int q_stride, OT* out, int out_stride, v
   const int waves = (splits == 1 && max_context > 512 && hd <= 64 && 16 * (32 + (size_t)hd * G) * sizeof(float) <= 65536) ? 16 : 4;
   const size_t lds = (size_t)waves * (32 + (size_t)hd * G) * sizeof(float);
   const dim3 grid(splits, nkv, n_decode), block(waves * 64);
-#define GB_CASE(HD)                                                                                                         \
-  if (hd == HD) {                                                                                                           \
-    if (waves == 16)                                                                                                        \
-      hipLaunchKernelGGL((decode_kernel<HD, 16, OT>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride, \
-                         (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
-                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits, ex);                       \
-    else                                                                                                                    \
-      hipLaunchKernelGGL((decode_kernel<HD, 4, OT>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride,  \
-                         (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,              \
-                         (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits, ex);                       \
+  // capped scores are a kernel of their own (bfloat16 results only), so that the others' score loops are what they were
+  constexpr bool kCanCap = std::is_same<OT, bf16>::value;
+  const bool cap = ex.softcap > 0.f;
+  GB_REQUIRE(!cap || kCanCap, "attention_decode: capped scores with float32 result rows are not served");
+#define GB_DECODE(HD, WAVES, CAP)                                                                                          \
+  hipLaunchKernelGGL((decode_kernel<HD, WAVES, OT, CAP>), grid, block, lds, stream, (const bf16*)q, q_stride, out, out_stride, \
+                     (float*)ws_acc, (float*)ws_ml, positions, tables, table_stride, (const bf16*)k_pages,                  \
+                     (const bf16*)v_pages, nh, nkv, page_size, scale, window, keep_first, chunk, splits, ex)
+#define GB_CASE(HD)                                                 \
+  if (hd == HD) {                                                   \
+    if (cap) {                                                      \
+      if constexpr (kCanCap) {                                      \
+        if (waves == 16) GB_DECODE(HD, 16, true);                   \
+        else GB_DECODE(HD, 4, true);                                \
+      }                                                             \
+    } else if (waves == 16) {                                       \
+      GB_DECODE(HD, 16, false);                                     \
+    } else {                                                        \
+      GB_DECODE(HD, 4, false);                                      \
+    }                                                               \
   }
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
+#undef GB_DECODE
   if (int rc = launched("attention_decode")) return rc;
   if (splits > 1) {
     GB_REQUIRE(splits <= 256, "attention_decode: %d chunks are more than the 256 the second pass combines", splits);
@@ -1040,11 +1055,23 @@ static int prefill_launch(const void* q, int q_stride, OT* out, int out_stride, 
     part_ml = part_ws + cells * hd;
   }
   const dim3 grid((max_q_len + 64 * per_group - 1) / (64 * per_group) * parts, nh, n_seqs), block(64 * per_group * split);
-#define GB_LAUNCH(HD, QB, PAIRS, SPLIT)                                                                                     \
-  hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT, OT>), grid, block, 0, stream, (const bf16*)q, q_stride, out, \
+  // capped scores are a kernel of their own (bfloat16 results only), so that the others' score loops are what they were
+  constexpr bool kCanCap = std::is_same<OT, bf16>::value;
+  const bool cap = ex.softcap > 0.f;
+  GB_REQUIRE(!cap || kCanCap, "attention_prefill: capped scores with float32 result rows are not served");
+#define GB_LAUNCH_AS(HD, QB, PAIRS, SPLIT, CAP)                                                                             \
+  hipLaunchKernelGGL((prefill_kernel<HD, QB, PAIRS, SPLIT, OT, CAP>), grid, block, 0, stream, (const bf16*)q, q_stride, out, \
                      out_stride, q_start, q_len, pos0, seq_base, tables, table_stride, (const bf16*)k_pages,               \
                      (const bf16*)v_pages, nh, nkv, page_shift, scale, window, keep_first, part_acc, part_ml, parts, first_row, \
                      n_rows, ex)
+#define GB_LAUNCH(HD, QB, PAIRS, SPLIT)                            \
+  do {                                                             \
+    if (cap) {                                                     \
+      if constexpr (kCanCap) GB_LAUNCH_AS(HD, QB, PAIRS, SPLIT, true); \
+    } else {                                                       \
+      GB_LAUNCH_AS(HD, QB, PAIRS, SPLIT, false);                   \
+    }                                                              \
+  } while (0)
 #define GB_CASE(HD)                                        \
   if (hd == HD) {                                          \
     if constexpr (HD <= 64) {                              \
@@ -1061,6 +1088,7 @@ static int prefill_launch(const void* q, int q_stride, OT* out, int out_stride, 
   GB_FOR_HEAD_SIZES(GB_CASE)
 #undef GB_CASE
 #undef GB_LAUNCH
+#undef GB_LAUNCH_AS
   if (int rc = launched("attention_prefill")) return rc;
   if (parts > 1) {
     hipLaunchKernelGGL(prefill_parts_kernel<OT>, dim3((unsigned)(n_rows * nh)), dim3((hd + 63) / 64 * 64), 0, stream, part_acc,
