@@ -127,10 +127,10 @@ def tekilix_like(shapes: dict, layers: int, run: int = 1024, experts: int = 8, t
     ff = shapes["intermediate_size"]
     moe = {"kind": "moe", "expert": {"ff": ff * 3 // 8 // 8 * 8}, "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}},
            "shared": {"ff": ff * 3 // 4 // 8 * 8}}
-    one = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 30.0,
-           "rot": {"dims": hd // 2, "base": 10000.0}, "mask": {"size": run}}
+    one = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "softcap": 50.0,
+           "rot": {"dims": hd // 2, "base": 100000.0}, "mask": {"size": run}}
     two = {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "conv": 4,
-           "rot": {"dims": hd // 2, "base": 250000.0, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}},
+           "rot": {"dims": hd // 2, "base": 500000.0, "scaling": {"factor": 8.0, "original": 2048, "fast": 16.0, "slow": 2.0}},
            "mask": {"size": run}}
     kinds = [{"type": "attention", "mixer": one, "mlp": moe}, {"type": "attention_2", "mixer": two, "mlp": moe}]
     return dict(architecture="Tekilix", vocab=shapes["vocab_size"], width=d, norm={"eps": shapes["rms_norm_eps"]},

@@ -97,8 +97,8 @@ def test_the_sink_takes_its_share_and_gives_nothing():
             assert p[h, i, :i + 1].tolist() == pytest.approx((e / (e.sum() + math.exp(float(sink[h])))).tolist())
             assert float(p[h, i, i + 1:].abs().sum()) == 0.0
     assert float(p[2].sum(-1).min()) == pytest.approx(1.0) and float(p[1].sum(-1).max()) < 0.95
-    assert float(pt.capped(torch.tensor(1000.0, dtype=F64), 30.0)) == pytest.approx(30.0)
-    assert float(pt.capped(torch.tensor(0.3, dtype=F64), 30.0)) == pytest.approx(30.0 * math.tanh(0.01))
+    assert float(pt.capped(torch.tensor(1000.0, dtype=F64), 25.0)) == pytest.approx(25.0)
+    assert float(pt.capped(torch.tensor(0.5, dtype=F64), 25.0)) == pytest.approx(25.0 * math.tanh(0.02))
     assert float(pt.capped(torch.tensor(5.0, dtype=F64), 0.0)) == 5.0
 
 
