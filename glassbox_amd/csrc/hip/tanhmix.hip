@@ -145,8 +145,8 @@ __global__ void qk_heads_kernel(
   int off = 0, first_pos = 0;
   float* st = nullptr;
   if (taps > 0) {
-    const int seq = tok_seq[t];
-    off = t - q_start[seq];
+    const int seq = single ? t : tok_seq[t];      // (every request one row: row t is request t's)
+    off = single ? 0 : t - q_start[seq];
     first_pos = pos0[seq];
     if (K > 0) st = state + (size_t)state_slots[seq] * K * channels;
   }
@@ -275,7 +275,8 @@ __global__ __launch_bounds__(256) void qk_heads_words_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = (float)x[e] + b[e];
   } else if (has) {
-    const int K = taps - 1, seq = tok_seq[t], off = t - q_start[seq], first_pos = pos0[seq];
+    // (every request one row: row t is request t's)
+    const int K = taps - 1, seq = single ? t : tok_seq[t], off = single ? 0 : t - q_start[seq], first_pos = pos0[seq];
     float* st = K > 0 ? state + (size_t)state_slots[seq] * K * channels + ch : nullptr;
     for (int jt = 0; jt < taps; ++jt) {
       const int back = K - jt;   // how many tokens before this one
